@@ -1,0 +1,234 @@
+#!/usr/bin/env python3
+"""Roofline benchmark of the depthwise oriented 1D convolution on one MI355X.
+
+A "step" is one pass of the hot path over one batch of synthetic input: fprop, dgrad and
+wgrad at each of the four ConvNeXt-T stage shapes (batch 64, K=31, theta_c = (c mod 8)*22.5
+degrees), i.e. 12 launches of the C-ABI entry points.  Inputs are resident in HBM before the
+timed region; buffer sets rotate so consecutive steps do not re-hit the 256 MB Infinity Cache.
+
+Prints ONE JSON line: `value` is the algorithmic GB/s of the whole step (sum of the 12
+operators' algorithmic bytes / step time); `detail` carries GB/s and the HBM-roofline
+fraction of every (shape, op); `roofline` is the dominant kernel (fprop at C=96, 56x56,
+the largest byte count), timed with events on the launch stream; `cpu_baseline` is the
+oracle's single-thread reference-order loops on a bounded sample of the same workload.
+"""
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E peak
+STAGES = [(96, 56), (192, 28), (384, 14), (768, 7)]
+BATCH, KSIZE = 64, 31
+ELEM = {"f32": 4, "bf16": 2, "f16": 2}
+
+
+def algorithmic_bytes(op, N, C, H, W, K, b, stride=1):
+    """Bytes an ideal implementation moves: each activation tensor once, plus weights and
+    the int8 tap table (fprop/dgrad) or the dw output (wgrad).  No halo re-reads, no
+    transposes, no reduction scratch."""
+    P, Q = -(-H // stride), -(-W // stride)
+    act = (N * C * H * W + N * C * P * Q) * b
+    if op == "wgrad":
+        return act + C * K * 4
+    return act + C * K * 4 + C * K * 2
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--dtype", default="f32", choices=list(ELEM))
+    ap.add_argument("--layout", default="nchw", choices=["nchw", "nhwc"])
+    ap.add_argument("--theta", default="roundrobin", choices=["roundrobin", "grouped"])
+    ap.add_argument("--kernel-iters", type=int, default=30,
+                    help="back-to-back launches per (shape, op) for the per-kernel timings")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--only", default="", help="restrict the per-kernel table, e.g. 96x56:fprop")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build measures one GPU only (the operator has no cross-GPU "
+              "exchange; see DESIGN.md on sharding); run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+
+    from oriented1d_amd import dwoconv1d as op
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(2)
+    dev = torch.device("cuda:0")
+    tdt = {"f32": torch.float32, "bf16": torch.bfloat16, "f16": torch.float16}[args.dtype]
+    b = ELEM[args.dtype]
+    nhwc = args.layout == "nhwc"
+
+    def theta_for(C):
+        if args.theta == "roundrobin":
+            return np.array([(c % 8) * math.pi / 8 for c in range(C)], dtype=np.float32)
+        return np.array([math.pi * (((8 * (c + 1) - 1) // C) / 8) for c in range(C)],
+                        dtype=np.float32)
+
+    # ------------------------------------------------------------------ resident inputs
+    g = torch.Generator(device=dev).manual_seed(0)
+    bytes_per_set = sum(3 * BATCH * C * HW * HW * b for C, HW in STAGES)
+    nsets = max(2, math.ceil(2 * 256e6 / (2 * BATCH * 96 * 56 * 56 * b)) + 1)
+    sets = []
+    for _ in range(nsets):
+        st = []
+        for C, HW in STAGES:
+            shape = (BATCH, HW, HW, C) if nhwc else (BATCH, C, HW, HW)
+            x = torch.randn(shape, device=dev, generator=g).to(tdt)
+            dy = torch.randn(shape, device=dev, generator=g).to(tdt)
+            w = torch.randn(C, 1, 1, KSIZE, device=dev, generator=g) * 0.02
+            taps = op.build_taps(torch.from_numpy(theta_for(C)), C, KSIZE).to(dev)
+            st.append((C, HW, x, dy, w, taps))
+        sets.append(st)
+
+    # Outputs and wgrad scratch are allocated once; the timed region holds nothing but the
+    # C-ABI calls (ctypes arguments are converted up front).
+    import ctypes
+
+    from oriented1d_amd import _lib
+    lib = _lib.load()
+    stream_h = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+    dt_code, lay_code = {"f32": 0, "bf16": 1, "f16": 2}[args.dtype], int(nhwc)
+    keep = []
+
+    def vp(t):
+        return ctypes.c_void_p(t.data_ptr())
+
+    calls = []  # calls[set][stage][op] -> zero-argument callable
+    for st in sets:
+        per_stage = []
+        for (C, HW, x, dy, w, taps) in st:
+            w2 = w.reshape(C, KSIZE).contiguous()
+            y = torch.empty_like(x)
+            dx = torch.empty_like(x)
+            dw = torch.empty(C, KSIZE, device=dev)
+            nb = lib.dwo_wgrad_scratch_bytes(BATCH, C, HW, HW, KSIZE, 1, dt_code, lay_code)
+            scr = torch.empty(max(nb, 16), dtype=torch.uint8, device=dev)
+            keep.extend([w2, y, dx, dw, scr])
+            dims = (BATCH, C, HW, HW, KSIZE, 1, dt_code, lay_code, stream_h)
+            fa = (vp(x), vp(w2), None, vp(taps), vp(y)) + dims
+            da = (vp(dy), vp(w2), vp(taps), vp(dx)) + dims
+            wa = (vp(dy), vp(x), vp(taps), vp(dw), None, vp(scr), nb) + dims
+            per_stage.append({
+                "fprop": (lambda a=fa: lib.dwo_fprop(*a)),
+                "dgrad": (lambda a=da: lib.dwo_dgrad(*a)),
+                "wgrad": (lambda a=wa: lib.dwo_wgrad(*a)),
+            })
+        calls.append(per_stage)
+    for per_stage in calls:  # one checked pass: any launch error surfaces here
+        for ops in per_stage:
+            for name, fn in ops.items():
+                _lib.check(fn(), "dwo_" + name)
+    torch.cuda.synchronize()
+
+    def run_op(name, si, i):
+        calls[i % nsets][si][name]()
+
+    def step(i):
+        for ops in calls[i % nsets]:
+            ops["fprop"]()
+            ops["dgrad"]()
+            ops["wgrad"]()
+
+    step_bytes = sum(algorithmic_bytes(o, BATCH, C, HW, HW, KSIZE, b)
+                     for C, HW in STAGES for o in ("fprop", "dgrad", "wgrad"))
+
+    # ------------------------------------------------------------------ timed steps
+    for i in range(args.warmup):
+        step(i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        step(i)
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    ms_per_step = (t1 - t0) * 1e3 / args.steps
+    value = step_bytes / (ms_per_step * 1e-3) / 1e9
+
+    # ------------------------------------------------------------------ per-kernel timings
+    # HIP events on the launch stream (torch's current stream is the one passed to the C ABI).
+    detail = {}
+    stream = torch.cuda.current_stream(dev)
+    for si, (C, HW) in enumerate(STAGES):
+        for name in ("fprop", "dgrad", "wgrad"):
+            key = "%dx%d:%s" % (C, HW, name)
+            if args.only and args.only != key:
+                continue
+            for i in range(3):
+                run_op(name, si, i)
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(stream)
+            for i in range(args.kernel_iters):
+                run_op(name, si, i)
+            e1.record(stream)
+            torch.cuda.synchronize()
+            us = e0.elapsed_time(e1) * 1e3 / args.kernel_iters
+            ab = algorithmic_bytes(name, BATCH, C, HW, HW, KSIZE, b)
+            gbs = ab / (us * 1e-6) / 1e9
+            detail[key] = {"us": round(us, 2), "GB/s": round(gbs, 1),
+                           "frac_hbm": round(gbs / HBM_PEAK_GBS, 4), "bytes": ab}
+
+    dom = detail.get("96x56:fprop")
+    roofline = None
+    if dom:
+        roofline = {"bound": "hbm", "kernel": "fprop C=96 56x56 N=64 %s %s" % (args.dtype, args.layout),
+                    "achieved": dom["GB/s"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                    "frac": round(dom["GB/s"] / HBM_PEAK_GBS, 4), "traffic": None,
+                    "launch_us": dom["us"], "algorithmic_bytes": dom["bytes"]}
+
+    # ------------------------------------------------------------------ CPU baseline (oracle)
+    cpu = None
+    if not args.no_cpu_baseline:
+        from oracle import dwo_oracle as oracle
+
+        rng = np.random.default_rng(0)
+        n_cpu = 4  # bounded sample: 4 of the 64 images at every stage shape, all three ops
+        cpu_bytes, cpu_s = 0, 0.0
+        for C, HW in STAGES:
+            th = theta_for(C)
+            x = rng.standard_normal((n_cpu, C, HW, HW)).astype(np.float32)
+            dy = rng.standard_normal((n_cpu, C, HW, HW)).astype(np.float32)
+            w = (rng.standard_normal((C, 1, 1, KSIZE)) * 0.02).astype(np.float32)
+            c0 = time.perf_counter()
+            oracle.fprop(x, w, th, acc="f32")
+            oracle.dgrad(dy, w, th, acc="f32")
+            oracle.wgrad(dy, x, th, KSIZE, acc="f32")
+            cpu_s += time.perf_counter() - c0
+            cpu_bytes += sum(algorithmic_bytes(o, n_cpu, C, HW, HW, KSIZE, 4)
+                             for o in ("fprop", "dgrad", "wgrad"))
+        cpu = {"value": round(cpu_bytes / cpu_s / 1e9, 4), "unit": "GB/s", "cores": 1,
+               "kind": "port",
+               "sample": "fp32 fprop+dgrad+wgrad, 4 of 64 images at each of the four stage "
+                         "shapes, single thread, reference loop order (%.1f s)" % cpu_s,
+               "host_cpus": os.cpu_count()}
+
+    out = {
+        "metric": "dwoconv1d fprop/dgrad/wgrad GB/s (% HBM peak); ConvNeXt-T-1D img/s",
+        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": args.dtype, "data": "synthetic",
+        "config": {"workload": "dwoconv1d fprop+dgrad+wgrad sweep at ConvNeXt-T stage shapes "
+                               "(C=96@56x56, 192@28x28, 384@14x14, 768@7x7), batch 64, K=31, "
+                               "8 orientations %s, stride 1" % args.theta,
+                   "layout": args.layout, "buffer_sets": nsets,
+                   "algorithmic_bytes_per_step": step_bytes},
+        "frac_hbm_peak": round(value / HBM_PEAK_GBS, 4),
+        "detail": detail, "roofline": roofline, "cpu_baseline": cpu,
+    }
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,112 @@
+/*
+ * libdwoconv1d_hip.so -- C ABI of the MI355X (gfx950) depthwise oriented 1D convolution.
+ *
+ * This is the boundary a binding of the reference's operator module would call in place
+ * of the five functions its JIT-built extension exports
+ * (models/dwoconv1d/dwoconv1d_kernel.py:29-36,54-60: fprop, dgrad, wgrad, nhwc_to_nchw,
+ * nchw_to_nhwc).  Plain pointers and sizes only; the library never allocates, frees or
+ * retains device memory: the caller owns inputs, outputs and scratch.  Every launch is
+ * asynchronous on the stream passed in (the reference launches on the current stream,
+ * models/dwoconv1d/kernels/kernels.cu:25).
+ *
+ * Operator definition (models/dwoconv1d_reference/kernels/kernels.cpp:36-52,71-90,111-126),
+ * pad = K/2, P = ceil(H/stride), Q = ceil(W/stride):
+ *   dh(s) = (int)(-sinf(theta_c) * (s - pad)),  dw(s) = (int)(cosf(theta_c) * (s - pad))
+ *   fprop: y[n,c,p,q]  = sum_s x[n,c,p*stride+dh(s),q*stride+dw(s)] * w[c,s]   (taps outside = 0)
+ *   dgrad: dx[n,c,h,w] = sum_s dy[n,c,(h-dh(s))/stride,(w-dw(s))/stride] * w[c,s]
+ *                        (only taps whose two numerators are divisible by stride and in range)
+ *   wgrad: dw[c,s]     = sum_{n,p,q} x[n,c,p*stride+dh(s),q*stride+dw(s)] * dy[n,c,p,q]
+ *
+ * Layouts: DWO_NCHW tensors are [N,C,H,W]; DWO_NHWC tensors are [N,H,W,C].  The NHWC entry
+ * points read and write NHWC directly, which replaces the reference's transpose passes
+ * (models/dwoconv1d/kernels/kernels.cu:56-68, nhwc_utils.h:46-110).
+ * Element types: activations x, y, dy, dx are fp32, bf16 or fp16; weights, bias, dw and db
+ * are always fp32 and all accumulation is fp32.
+ */
+#ifndef DWOCONV1D_HIP_H
+#define DWOCONV1D_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* status codes: 0 ok, negative = argument error, positive = hipError_t of the launch */
+#define DWO_OK 0
+#define DWO_ERR_NULL_POINTER (-1)
+#define DWO_ERR_BAD_SHAPE (-2)    /* N,C,H,W < 1 or sizes overflow int32 indexing */
+#define DWO_ERR_BAD_KERNEL (-3)   /* K even, < 1 or > DWO_MAX_K */
+#define DWO_ERR_BAD_STRIDE (-4)   /* stride not in {1,2,4} */
+#define DWO_ERR_BAD_DTYPE (-5)
+#define DWO_ERR_BAD_LAYOUT (-6)
+#define DWO_ERR_SCRATCH_TOO_SMALL (-7)
+#define DWO_ERR_BAD_TAPS (-8)     /* host-side tap blob does not match C,K */
+
+#define DWO_MAX_K 63
+
+#define DWO_F32 0
+#define DWO_BF16 1
+#define DWO_F16 2
+
+#define DWO_NCHW 0
+#define DWO_NHWC 1
+
+/* Library version (major*10000 + minor*100 + patch). */
+int dwo_version(void);
+
+/* Human-readable text for a status returned by any entry point. */
+const char *dwo_status_string(int status);
+
+/*
+ * Host-side tap table.  Replaces the per-thread sincosf + truncation of the reference
+ * kernels (models/dwoconv1d/kernels/kernels.h:240-241,285-287) with one table computed
+ * on the host in fp32 exactly as kernels.cpp:37,43-44 does.  `theta_host` holds C angles
+ * in radians.  The caller copies the `dwo_taps_bytes(C,K)`-byte blob to device memory and
+ * passes that device pointer as `taps` below; the blob's layout is private to the library.
+ */
+size_t dwo_taps_bytes(int C, int K);
+int dwo_build_taps(const float *theta_host, int C, int K, void *taps_host);
+
+/* Debug/inspection helper: (dh,dw) of channel c, tap s from a host blob. */
+int dwo_taps_get(const void *taps_host, int c, int s, int *dh, int *dw);
+
+/*
+ * fprop -- replaces `fprop(x, w, theta)` (models/dwoconv1d/kernels/kernels.cu:15-27) plus
+ * the separate bias add of models/dwoconv1d/dwoconv1d.py:34-35 when `bias` is non-NULL.
+ * x: [N,C,H,W] or [N,H,W,C] `dtype`; w: [C,K] fp32; bias: [C] fp32 or NULL;
+ * y: [N,C,P,Q] or [N,P,Q,C] `dtype`.
+ */
+int dwo_fprop(const void *x, const float *w, const float *bias, const void *taps, void *y,
+              int N, int C, int H, int W, int K, int stride, int dtype, int layout,
+              void *stream);
+
+/*
+ * dgrad -- replaces `dgrad(dy, w, theta)` (models/dwoconv1d/kernels/kernels.cu:29-40).
+ * dy: [N,C,P,Q] / [N,P,Q,C]; dx: [N,C,H,W] / [N,H,W,C]; H,W are the input extents.
+ */
+int dwo_dgrad(const void *dy, const float *w, const void *taps, void *dx,
+              int N, int C, int H, int W, int K, int stride, int dtype, int layout,
+              void *stream);
+
+/*
+ * wgrad -- replaces `wgrad(dy, x, theta)` (models/dwoconv1d/kernels/kernels.cu:42-54) and,
+ * when `db` is non-NULL, the bias gradient `dy.sum([0,2,3])` of dwoconv1d.py:66-67.
+ * Two-stage and deterministic: workgroups write partial sums into `scratch`
+ * (`dwo_wgrad_scratch_bytes` bytes, caller-allocated, contents undefined on entry and
+ * exit) and one second-stage kernel reduces them in a fixed order -- no atomics, unlike
+ * models/dwoconv1d/kernels/kernels.h:504-517.  dw: [C,K] fp32 (fully overwritten);
+ * db: [C] fp32 or NULL.
+ */
+size_t dwo_wgrad_scratch_bytes(int N, int C, int H, int W, int K, int stride, int dtype,
+                               int layout);
+int dwo_wgrad(const void *dy, const void *x, const void *taps, float *dw, float *db,
+              void *scratch, size_t scratch_bytes,
+              int N, int C, int H, int W, int K, int stride, int dtype, int layout,
+              void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DWOCONV1D_HIP_H */

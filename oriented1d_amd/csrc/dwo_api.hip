@@ -1,0 +1,228 @@
+// C ABI of libdwoconv1d_hip.so: argument validation, host-side tap table, kernel selection
+// and launch.  No device allocation, no retained pointers, no global mutable state.
+#include <math.h>
+#include <string.h>
+
+#include "dwo_common.h"
+#include "dwo_generic.h"
+
+using namespace dwo;
+
+namespace {
+
+int log2_stride(int stride) { return stride == 1 ? 0 : (stride == 2 ? 1 : (stride == 4 ? 2 : -1)); }
+
+int check_common(int N, int C, int H, int W, int K, int stride, int dtype, int layout) {
+    if (N < 1 || C < 1 || H < 1 || W < 1) return DWO_ERR_BAD_SHAPE;
+    if ((double)N * C * H * W >= 2147483648.0) return DWO_ERR_BAD_SHAPE;
+    if (K < 1 || K > DWO_MAX_K || (K & 1) == 0) return DWO_ERR_BAD_KERNEL;
+    if (log2_stride(stride) < 0) return DWO_ERR_BAD_STRIDE;
+    if (dtype != DWO_F32 && dtype != DWO_BF16 && dtype != DWO_F16) return DWO_ERR_BAD_DTYPE;
+    if (layout != DWO_NCHW && layout != DWO_NHWC) return DWO_ERR_BAD_LAYOUT;
+    return DWO_OK;
+}
+
+ConvDims make_dims(int N, int C, int H, int W, int K, int stride) {
+    ConvDims d;
+    d.N = N, d.C = C, d.H = H, d.W = W, d.K = K, d.stride = stride;
+    d.shift = log2_stride(stride);
+    d.P = (H + stride - 1) / stride;
+    d.Q = (W + stride - 1) / stride;
+    return d;
+}
+
+int launch_status() {
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? DWO_OK : (int)e;
+}
+
+struct WgradSplit {
+    int blocks_x, G, per_slice;
+};
+
+// Slices of the N*P*Q positions per channel block for the generic wgrad: enough workgroups
+// to fill 256 CUs several times over, at least 1024 positions per slice.
+WgradSplit wgrad_generic_split(const ConvDims &d, int layout) {
+    WgradSplit s;
+    s.blocks_x = layout == DWO_NCHW ? d.C : (d.C + 63) / 64;
+    const long npos = (long)d.N * d.P * d.Q;
+    long G = 4096 / s.blocks_x;
+    const long cap = (npos + 1023) / 1024;
+    if (G > cap) G = cap;
+    if (G < 1) G = 1;
+    s.per_slice = (int)((npos + G - 1) / G);
+    s.G = (int)((npos + s.per_slice - 1) / s.per_slice);
+    return s;
+}
+
+template <typename T>
+int fprop_t(const void *x, const float *w, const float *bias, const void *taps, void *y,
+            const ConvDims &d, int layout, hipStream_t st) {
+    const int total = d.N * d.C * d.P * d.Q;
+    const dim3 grid((total + 255) / 256), block(256);
+    const int8_t *tp = taps_dhdw(taps);
+    if (layout == DWO_NCHW)
+        gather_generic_kernel<T, DWO_NCHW, false><<<grid, block, 0, st>>>(
+            (const T *)x, w, bias, tp, (T *)y, d, total);
+    else
+        gather_generic_kernel<T, DWO_NHWC, false><<<grid, block, 0, st>>>(
+            (const T *)x, w, bias, tp, (T *)y, d, total);
+    return launch_status();
+}
+
+template <typename T>
+int dgrad_t(const void *dy, const float *w, const void *taps, void *dx, const ConvDims &d,
+            int layout, hipStream_t st) {
+    const int total = d.N * d.C * d.H * d.W;
+    const dim3 grid((total + 255) / 256), block(256);
+    const int8_t *tp = taps_dhdw(taps);
+    if (layout == DWO_NCHW)
+        gather_generic_kernel<T, DWO_NCHW, true><<<grid, block, 0, st>>>(
+            (const T *)dy, w, nullptr, tp, (T *)dx, d, total);
+    else
+        gather_generic_kernel<T, DWO_NHWC, true><<<grid, block, 0, st>>>(
+            (const T *)dy, w, nullptr, tp, (T *)dx, d, total);
+    return launch_status();
+}
+
+template <typename T>
+int wgrad_t(const void *dy, const void *x, const void *taps, float *dw, float *db, void *scratch,
+            const ConvDims &d, int layout, hipStream_t st) {
+    const WgradSplit s = wgrad_generic_split(d, layout);
+    const dim3 grid(s.blocks_x, s.G), block(256);
+    const int8_t *tp = taps_dhdw(taps);
+    float *part = (float *)scratch;
+    if (layout == DWO_NCHW)
+        wgrad_generic_kernel<T, DWO_NCHW><<<grid, block, 0, st>>>((const T *)dy, (const T *)x, tp,
+                                                                  part, d, s.G, s.per_slice);
+    else
+        wgrad_generic_kernel<T, DWO_NHWC><<<grid, block, 0, st>>>((const T *)dy, (const T *)x, tp,
+                                                                  part, d, s.G, s.per_slice);
+    int rc = launch_status();
+    if (rc != DWO_OK) return rc;
+    const int cells = d.C * (d.K + 1);
+    wgrad_reduce_kernel<<<dim3((cells + 255) / 256), dim3(256), 0, st>>>(part, dw, db, d.C, d.K,
+                                                                        s.G);
+    return launch_status();
+}
+
+}  // namespace
+
+extern "C" {
+
+int dwo_version(void) { return 100; }
+
+const char *dwo_status_string(int status) {
+    switch (status) {
+        case DWO_OK: return "ok";
+        case DWO_ERR_NULL_POINTER: return "null pointer argument";
+        case DWO_ERR_BAD_SHAPE: return "invalid tensor extents (must be >= 1 and index in int32)";
+        case DWO_ERR_BAD_KERNEL: return "kernel size must be odd and in [1, 63]";
+        case DWO_ERR_BAD_STRIDE: return "stride must be 1, 2 or 4";
+        case DWO_ERR_BAD_DTYPE: return "unsupported element type";
+        case DWO_ERR_BAD_LAYOUT: return "unsupported layout";
+        case DWO_ERR_SCRATCH_TOO_SMALL: return "wgrad scratch buffer too small";
+        case DWO_ERR_BAD_TAPS: return "tap table does not match C and K";
+        default: break;
+    }
+    if (status > 0) return hipGetErrorString((hipError_t)status);
+    return "unknown status";
+}
+
+size_t dwo_taps_bytes(int C, int K) {
+    if (C < 1 || K < 1 || K > DWO_MAX_K || (K & 1) == 0) return 0;
+    return kTapsHeaderBytes + taps_dhdw_bytes(C, K) + (((size_t)C * 4 + 15) & ~(size_t)15);
+}
+
+int dwo_build_taps(const float *theta_host, int C, int K, void *taps_host) {
+    if (theta_host == nullptr || taps_host == nullptr) return DWO_ERR_NULL_POINTER;
+    if (C < 1) return DWO_ERR_BAD_SHAPE;
+    if (K < 1 || K > DWO_MAX_K || (K & 1) == 0) return DWO_ERR_BAD_KERNEL;
+    memset(taps_host, 0, dwo_taps_bytes(C, K));
+    int32_t *hdr = (int32_t *)taps_host;
+    hdr[0] = kTapsMagic, hdr[1] = kTapsVersion, hdr[2] = C, hdr[3] = K;
+    hdr[4] = kTapsHeaderBytes;
+    hdr[5] = kTapsHeaderBytes + (int32_t)taps_dhdw_bytes(C, K);
+    int8_t *dhdw = (int8_t *)taps_host + kTapsHeaderBytes;
+    int32_t *cls = (int32_t *)((int8_t *)taps_host + hdr[5]);
+    const int pad = K / 2;
+    for (int c = 0; c < C; c++) {
+        // models/dwoconv1d_reference/kernels/kernels.cpp:37,43-44: fp32 sine and cosine, a
+        // float product, and a C cast to int (truncation toward zero).
+        const float sin_ = sinf(theta_host[c]), cos_ = cosf(theta_host[c]);
+        for (int s = 0; s < K; s++) {
+            volatile float fh = -sin_ * (float)(s - pad);
+            volatile float fw = cos_ * (float)(s - pad);
+            dhdw[((size_t)c * K + s) * 2 + 0] = (int8_t)(int)fh;
+            dhdw[((size_t)c * K + s) * 2 + 1] = (int8_t)(int)fw;
+        }
+        cls[c] = -1;
+    }
+    return DWO_OK;
+}
+
+int dwo_taps_get(const void *taps_host, int c, int s, int *dh, int *dw) {
+    if (taps_host == nullptr || dh == nullptr || dw == nullptr) return DWO_ERR_NULL_POINTER;
+    const int32_t *hdr = (const int32_t *)taps_host;
+    if (hdr[0] != kTapsMagic || hdr[1] != kTapsVersion) return DWO_ERR_BAD_TAPS;
+    if (c < 0 || c >= hdr[2] || s < 0 || s >= hdr[3]) return DWO_ERR_BAD_SHAPE;
+    const int8_t *dhdw = taps_dhdw(taps_host);
+    *dh = dhdw[((size_t)c * hdr[3] + s) * 2];
+    *dw = dhdw[((size_t)c * hdr[3] + s) * 2 + 1];
+    return DWO_OK;
+}
+
+int dwo_fprop(const void *x, const float *w, const float *bias, const void *taps, void *y, int N,
+              int C, int H, int W, int K, int stride, int dtype, int layout, void *stream) {
+    int rc = check_common(N, C, H, W, K, stride, dtype, layout);
+    if (rc != DWO_OK) return rc;
+    if (!x || !w || !taps || !y) return DWO_ERR_NULL_POINTER;
+    const ConvDims d = make_dims(N, C, H, W, K, stride);
+    hipStream_t st = (hipStream_t)stream;
+    switch (dtype) {
+        case DWO_F32: return fprop_t<float>(x, w, bias, taps, y, d, layout, st);
+        case DWO_BF16: return fprop_t<bf16_t>(x, w, bias, taps, y, d, layout, st);
+        default: return fprop_t<f16_t>(x, w, bias, taps, y, d, layout, st);
+    }
+}
+
+int dwo_dgrad(const void *dy, const float *w, const void *taps, void *dx, int N, int C, int H,
+              int W, int K, int stride, int dtype, int layout, void *stream) {
+    int rc = check_common(N, C, H, W, K, stride, dtype, layout);
+    if (rc != DWO_OK) return rc;
+    if (!dy || !w || !taps || !dx) return DWO_ERR_NULL_POINTER;
+    const ConvDims d = make_dims(N, C, H, W, K, stride);
+    hipStream_t st = (hipStream_t)stream;
+    switch (dtype) {
+        case DWO_F32: return dgrad_t<float>(dy, w, taps, dx, d, layout, st);
+        case DWO_BF16: return dgrad_t<bf16_t>(dy, w, taps, dx, d, layout, st);
+        default: return dgrad_t<f16_t>(dy, w, taps, dx, d, layout, st);
+    }
+}
+
+size_t dwo_wgrad_scratch_bytes(int N, int C, int H, int W, int K, int stride, int dtype,
+                               int layout) {
+    if (check_common(N, C, H, W, K, stride, dtype, layout) != DWO_OK) return 0;
+    const ConvDims d = make_dims(N, C, H, W, K, stride);
+    const WgradSplit s = wgrad_generic_split(d, layout);
+    return (size_t)C * (K + 1) * s.G * sizeof(float);
+}
+
+int dwo_wgrad(const void *dy, const void *x, const void *taps, float *dw, float *db,
+              void *scratch, size_t scratch_bytes, int N, int C, int H, int W, int K, int stride,
+              int dtype, int layout, void *stream) {
+    int rc = check_common(N, C, H, W, K, stride, dtype, layout);
+    if (rc != DWO_OK) return rc;
+    if (!dy || !x || !taps || !dw || !scratch) return DWO_ERR_NULL_POINTER;
+    if (scratch_bytes < dwo_wgrad_scratch_bytes(N, C, H, W, K, stride, dtype, layout))
+        return DWO_ERR_SCRATCH_TOO_SMALL;
+    const ConvDims d = make_dims(N, C, H, W, K, stride);
+    hipStream_t st = (hipStream_t)stream;
+    switch (dtype) {
+        case DWO_F32: return wgrad_t<float>(dy, x, taps, dw, db, scratch, d, layout, st);
+        case DWO_BF16: return wgrad_t<bf16_t>(dy, x, taps, dw, db, scratch, d, layout, st);
+        default: return wgrad_t<f16_t>(dy, x, taps, dw, db, scratch, d, layout, st);
+    }
+}
+
+}  // extern "C"

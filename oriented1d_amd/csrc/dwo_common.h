@@ -1,0 +1,84 @@
+// Shared device/host helpers for the gfx950 depthwise oriented 1D convolution kernels.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "dwoconv1d_hip.h"
+
+namespace dwo {
+
+// ---------------------------------------------------------------------------------------------
+// Tap blob (private layout).  Built on the host by dwo_build_taps, copied verbatim to the device.
+//   int32 header[8] : magic, version, C, K, off_dhdw, off_class, 0, 0
+//   int8  dhdw[C][K][2]        (dh, dw) of every tap, padded to 16 bytes
+//   int32 cls[C]               canonical orientation id 0..7 of the channel's tap pattern
+//                              (k * 22.5 degrees), or -1 when the pattern is not canonical
+// ---------------------------------------------------------------------------------------------
+constexpr int32_t kTapsMagic = 0x44574f31;  // "DWO1"
+constexpr int32_t kTapsVersion = 2;
+constexpr int kTapsHeaderInts = 8;
+constexpr int kTapsHeaderBytes = kTapsHeaderInts * 4;
+
+__host__ __device__ inline size_t taps_dhdw_bytes(int C, int K) {
+    return (((size_t)C * K * 2) + 15) & ~(size_t)15;
+}
+__host__ __device__ inline const int8_t *taps_dhdw(const void *blob) {
+    return reinterpret_cast<const int8_t *>(blob) + kTapsHeaderBytes;
+}
+__host__ __device__ inline const int32_t *taps_class(const void *blob, int C, int K) {
+    return reinterpret_cast<const int32_t *>(reinterpret_cast<const int8_t *>(blob) +
+                                             kTapsHeaderBytes + taps_dhdw_bytes(C, K));
+}
+
+// ---------------------------------------------------------------------------------------------
+// Element types.  Activations are fp32, bf16 (raw uint16 bits) or fp16; arithmetic is fp32.
+// ---------------------------------------------------------------------------------------------
+struct bf16_t {
+    uint16_t bits;
+};
+typedef _Float16 f16_t;
+
+__device__ __forceinline__ float to_float(float v) { return v; }
+__device__ __forceinline__ float to_float(bf16_t v) {
+    return __uint_as_float(static_cast<uint32_t>(v.bits) << 16);
+}
+__device__ __forceinline__ float to_float(f16_t v) { return static_cast<float>(v); }
+
+template <typename T>
+__device__ __forceinline__ T from_float(float v);
+template <>
+__device__ __forceinline__ float from_float<float>(float v) {
+    return v;
+}
+template <>
+__device__ __forceinline__ bf16_t from_float<bf16_t>(float v) {
+    // round to nearest even; NaN stays NaN (quiet)
+    uint32_t u = __float_as_uint(v);
+    bf16_t r;
+    if ((u & 0x7fffffffu) > 0x7f800000u) {
+        r.bits = static_cast<uint16_t>((u >> 16) | 0x0040u);
+    } else {
+        u += 0x7fffu + ((u >> 16) & 1u);
+        r.bits = static_cast<uint16_t>(u >> 16);
+    }
+    return r;
+}
+template <>
+__device__ __forceinline__ f16_t from_float<f16_t>(float v) {
+    return static_cast<f16_t>(v);
+}
+
+// Wave64 sum via cross-lane shuffles; every lane ends with the total of lanes >= itself folded
+// down, lane 0 holds the wave total.
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_down(v, off, 64);
+    return v;
+}
+
+struct ConvDims {
+    int N, C, H, W, P, Q, K, stride, shift;  // shift = log2(stride)
+};
+
+}  // namespace dwo

@@ -1,0 +1,314 @@
+"""Depthwise oriented 1D convolution operator module for MI355X.
+
+Host-side mirror of the reference's operator module (models/dwoconv1d/dwoconv1d.py): same
+class names, constructor, parameters (``weight [C,1,1,K]``, ``bias [C]``, ``theta``),
+attributes and autograd contract, so ``models/convnext.py:115-127`` can construct it
+unchanged.  All arithmetic happens in ``libdwoconv1d_hip.so`` through the C ABI declared
+in ``include/dwoconv1d_hip.h``; tensors here only provide device memory and the stream.
+
+Differences from the reference, all supersets:
+* bf16/fp16 activations are computed (fp32 accumulate) instead of being reinterpreted as
+  float (reference: kernels.cu:25 casts the pointer whatever the dtype).
+* ``nhwc=True`` runs NHWC-native kernels; no transposed copies are made
+  (reference: dwoconv1d.py:25-26,36-37,50-51,58-59).
+* bias add is fused into fprop and the bias gradient into wgrad
+  (reference: dwoconv1d.py:34-35,66-67).
+* ``arbitrary_size=True`` needs no pad-to-power-of-two / crop round trip
+  (reference: dwoconv1d.py:154-187); the kernels take any H, W and give
+  ceil(H/stride) x ceil(W/stride) outputs, the same values that path produces.
+"""
+import ctypes
+
+import numpy as np
+import torch
+import torch.nn as nn
+
+from . import _lib
+
+__all__ = ["DepthwiseOrientedConv1d"]
+
+_DTYPES = {torch.float32: _lib.F32, torch.bfloat16: _lib.BF16, torch.float16: _lib.F16}
+
+
+def _ptr(t):
+    return ctypes.c_void_p(t.data_ptr()) if t is not None else None
+
+
+def _stream(t):
+    return ctypes.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
+
+
+def _check_activation(t, name):
+    # models/dwoconv1d/kernels/kernels.cu:11-13,17-18
+    if not t.is_cuda:
+        raise RuntimeError("%s must be a CUDA tensor" % name)
+    if not t.is_contiguous():
+        raise RuntimeError("%s must be contiguous" % name)
+    if t.dtype not in _DTYPES:
+        raise RuntimeError("%s has unsupported dtype %s" % (name, t.dtype))
+    if t.dim() != 4:
+        raise RuntimeError("%s must be a 4-d tensor" % name)
+
+
+def build_taps(theta, C, K):
+    """Host tap table for ``theta`` ([C] or [C,1] radians) as a uint8 CPU tensor.
+
+    The table is computed by the library on the host in fp32
+    (models/dwoconv1d_reference/kernels/kernels.cpp:37,43-44)."""
+    lib = _lib.load()
+    th = theta.detach().to(device="cpu", dtype=torch.float32).reshape(-1).contiguous()
+    if th.numel() != C:
+        raise RuntimeError("theta must hold one angle per channel (%d), got %d" % (C, th.numel()))
+    blob = torch.empty(lib.dwo_taps_bytes(C, K), dtype=torch.uint8)
+    _lib.check(lib.dwo_build_taps(_ptr(th), C, K, _ptr(blob)), "dwo_build_taps")
+    return blob
+
+
+def taps_to_numpy(blob, C, K):
+    """(dh, dw) int arrays [C,K] read back from a host tap blob (inspection / tests)."""
+    lib = _lib.load()
+    dh, dw = np.empty((C, K), np.int32), np.empty((C, K), np.int32)
+    a, b = ctypes.c_int(), ctypes.c_int()
+    for c in range(C):
+        for s in range(K):
+            _lib.check(lib.dwo_taps_get(_ptr(blob), c, s, ctypes.byref(a), ctypes.byref(b)),
+                       "dwo_taps_get")
+            dh[c, s], dw[c, s] = a.value, b.value
+    return dh, dw
+
+
+class _TapCache:
+    """Device tap table of one theta tensor, rebuilt when theta is modified or moved."""
+
+    def __init__(self):
+        self.key = None
+        self.dev = None
+
+    def get(self, theta, C, K, device):
+        key = (theta.data_ptr(), theta._version, str(device), C, K)
+        if key != self.key:
+            self.dev = build_taps(theta, C, K).to(device)
+            self.key = key
+        return self.dev
+
+
+def _dims(x, nhwc):
+    if nhwc:
+        N, H, W, C = x.shape
+    else:
+        N, C, H, W = x.shape
+    return N, C, H, W
+
+
+def _out_shape(N, C, H, W, stride, nhwc):
+    P, Q = -(-H // stride), -(-W // stride)
+    return (N, P, Q, C) if nhwc else (N, C, P, Q)
+
+
+def _w2d(w, C):
+    w = w.detach().reshape(C, -1)
+    return w.to(torch.float32).contiguous()
+
+
+def fprop(x, w, taps, stride=1, bias=None, nhwc=False):
+    """y = fprop(x, w, theta) (+ bias).  x: [N,C,H,W] or [N,H,W,C]; w: [C,1,1,K]."""
+    lib = _lib.load()
+    _check_activation(x, "x")
+    N, C, H, W = _dims(x, nhwc)
+    w2 = _w2d(w, C)
+    K = w2.shape[1]
+    b = bias.detach().to(torch.float32).contiguous() if bias is not None else None
+    y = torch.empty(_out_shape(N, C, H, W, stride, nhwc), dtype=x.dtype, device=x.device)
+    _lib.check(lib.dwo_fprop(_ptr(x), _ptr(w2), _ptr(b), _ptr(taps), _ptr(y), N, C, H, W, K,
+                             stride, _DTYPES[x.dtype], int(nhwc), _stream(x)), "dwo_fprop")
+    return y
+
+
+def dgrad(dy, w, taps, in_hw, stride=1, nhwc=False):
+    """dx = dgrad(dy, w, theta); ``in_hw`` is the (H, W) of the forward input."""
+    lib = _lib.load()
+    _check_activation(dy, "dy")
+    H, W = in_hw
+    N, C, P, Q = _dims(dy, nhwc)
+    if (P, Q) != (-(-H // stride), -(-W // stride)):
+        raise RuntimeError("dy extent does not match the input extent and stride")
+    w2 = _w2d(w, C)
+    K = w2.shape[1]
+    dx = torch.empty((N, H, W, C) if nhwc else (N, C, H, W), dtype=dy.dtype, device=dy.device)
+    _lib.check(lib.dwo_dgrad(_ptr(dy), _ptr(w2), _ptr(taps), _ptr(dx), N, C, H, W, K, stride,
+                             _DTYPES[dy.dtype], int(nhwc), _stream(dy)), "dwo_dgrad")
+    return dx
+
+
+def wgrad(dy, x, taps, K, stride=1, nhwc=False, with_bias=False):
+    """(dw [C,1,1,K] fp32, db [C] fp32 or None) = wgrad(dy, x, theta)."""
+    lib = _lib.load()
+    _check_activation(dy, "dy")
+    _check_activation(x, "x")
+    if dy.dtype != x.dtype:
+        raise RuntimeError("dy and x must have the same dtype")
+    N, C, H, W = _dims(x, nhwc)
+    if tuple(dy.shape) != _out_shape(N, C, H, W, stride, nhwc):
+        raise RuntimeError("dy extent does not match the input extent and stride")
+    dt, lay = _DTYPES[x.dtype], int(nhwc)
+    nbytes = lib.dwo_wgrad_scratch_bytes(N, C, H, W, K, stride, dt, lay)
+    scratch = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=x.device)
+    dw = torch.empty((C, 1, 1, K), dtype=torch.float32, device=x.device)
+    db = torch.empty((C,), dtype=torch.float32, device=x.device) if with_bias else None
+    _lib.check(lib.dwo_wgrad(_ptr(dy), _ptr(x), _ptr(taps), _ptr(dw), _ptr(db), _ptr(scratch),
+                             nbytes, N, C, H, W, K, stride, dt, lay, _stream(x)), "dwo_wgrad")
+    return dw, db
+
+
+class _DepthwiseOrientedConv1d(torch.autograd.Function):
+    """Autograd contract of models/dwoconv1d/dwoconv1d.py:18-69.
+
+    ``apply(x, w, theta, bias, module, nhwc, resid)``; ``module`` is the owning
+    ``DepthwiseOrientedConv1d`` (the reference passes its tuple of compiled functions in
+    this slot).  backward returns (dx, dw, None, db, None, None, None): theta never
+    receives a gradient (dwoconv1d.py:64)."""
+
+    @staticmethod
+    def forward(ctx, x, w, theta, bias, module, nhwc=False, resid=None):
+        stride = module.stride[0]
+        C = w.shape[0]
+        K = w.shape[-1]
+        w_eff = w.detach().to(torch.float32)
+        if resid is not None:
+            w_eff = w_eff + resid.to(w_eff)
+        x = x.contiguous()
+        _check_activation(x, "x")
+        N, Cx, H, W = _dims(x, nhwc)
+        if Cx != C:
+            raise RuntimeError("input has %d channels, weight has %d" % (Cx, C))
+        if not module.arbitrary_size and (H % stride != 0 or W % stride != 0):
+            # models/dwoconv1d/kernels/kernels.cu:20
+            raise RuntimeError("Invalid input size: H,W not divisible by stride")
+        taps = module._taps.get(theta, C, K, x.device)
+
+        ctx.set_materialize_grads(False)
+        ctx.stride, ctx.nhwc, ctx.K = stride, nhwc, K
+        ctx.with_bias = bias is not None
+        ctx.w_dtype = w.dtype
+        ctx.b_dtype = bias.dtype if bias is not None else None
+        ctx.save_for_backward(x, w_eff, taps)
+        return fprop(x, w_eff, taps, stride, bias=bias, nhwc=nhwc)
+
+    @staticmethod
+    def backward(ctx, dy):
+        if dy is None:
+            return None, None, None, None, None, None, None
+        x, w_eff, taps = ctx.saved_tensors
+        dy = dy.contiguous()
+        if dy.dtype != x.dtype:
+            dy = dy.to(x.dtype)
+        N, C, H, W = _dims(x, ctx.nhwc)
+        dx = dw = db = None
+        if ctx.needs_input_grad[0]:
+            dx = dgrad(dy, w_eff, taps, (H, W), ctx.stride, nhwc=ctx.nhwc)
+        need_db = ctx.with_bias and ctx.needs_input_grad[3]
+        if ctx.needs_input_grad[1]:
+            dw, db32 = wgrad(dy, x, taps, ctx.K, ctx.stride, nhwc=ctx.nhwc, with_bias=need_db)
+            dw = dw.to(ctx.w_dtype)
+            if need_db:
+                db = db32.to(ctx.b_dtype)
+        elif need_db:
+            red = [0, 1, 2] if ctx.nhwc else [0, 2, 3]
+            db = dy.sum(dim=red, dtype=torch.float32).to(ctx.b_dtype)
+        return dx, dw, None, db, None, None, None
+
+
+def oriented_dwconv1d_get_module_from_params(ftype, kernel_size, stride, pad, Sb=None):
+    """Five-function tuple in the reference's order (models/dwoconv1d/dwoconv1d.py:72-80):
+    (fprop(x,w,theta), dgrad(dy,w,theta), wgrad(dy,x,theta), nhwc_to_nchw, nchw_to_nhwc),
+    all on NCHW tensors.  ``ftype``, ``pad`` and ``Sb`` are accepted for signature
+    compatibility: there is nothing to compile per configuration, pad is always
+    ``kernel_size // 2`` and the kernels need no filter partitioning."""
+    K = int(kernel_size)
+    stride = int(stride)
+
+    def _taps(theta, C, dev):
+        return build_taps(theta, C, K).to(dev)
+
+    def f(x, w, theta):
+        return fprop(x, w, _taps(theta, x.shape[1], x.device), stride)
+
+    def d(dy, w, theta):
+        hw = (dy.shape[2] * stride, dy.shape[3] * stride)
+        return dgrad(dy, w, _taps(theta, dy.shape[1], dy.device), hw, stride)
+
+    def g(dy, x, theta):
+        return wgrad(dy, x, _taps(theta, x.shape[1], x.device), K, stride)[0].to(x.dtype)
+
+    def nhwc_to_nchw(x):
+        return x.permute(0, 3, 1, 2).contiguous()
+
+    def nchw_to_nhwc(x):
+        return x.permute(0, 2, 3, 1).contiguous()
+
+    return f, d, g, nhwc_to_nchw, nchw_to_nhwc
+
+
+class DepthwiseOrientedConv1d(nn.Conv2d):
+    """Drop-in for models/dwoconv1d/dwoconv1d.py:92-198.
+
+    ``padding`` only shapes the parent ``nn.Conv2d``; the compute path always pads by
+    ``kernel_size // 2`` (dwoconv1d.py:133)."""
+
+    def __init__(
+        self,
+        in_channels,
+        out_channels,
+        kernel_size=3,
+        *,
+        groups=1,
+        stride=1,
+        padding=1,
+        bias=True,
+        angle=0,
+        nhwc=False,
+        resid=False,
+        arbitrary_size=False,
+    ):
+        super().__init__(
+            in_channels,
+            out_channels,
+            (1, kernel_size),
+            groups=groups,
+            stride=stride,
+            padding=(0, padding),
+            bias=bias,
+        )
+        assert (
+            isinstance(kernel_size, int)
+            and in_channels == out_channels
+            and groups == in_channels
+            and kernel_size % 2 == 1
+        )
+        assert self.stride[0] == self.stride[1]
+        assert kernel_size <= 63 and self.stride[0] in (1, 2, 4)
+
+        if isinstance(angle, (float, int)):
+            angle = torch.zeros((in_channels, 1)) + angle
+        self.theta = nn.Parameter(torch.as_tensor(angle, dtype=torch.float32).clone(),
+                                  requires_grad=True)
+        self.nhwc = nhwc
+        self.arbitrary_size = arbitrary_size
+        pad = kernel_size // 2
+        if resid:
+            onehot = torch.zeros_like(self.weight.detach())
+            onehot[:, :, :, pad:pad + 1] = 1
+            # follows .to()/.cuda() with the module, not part of the state_dict
+            self.register_buffer("resid", onehot, persistent=False)
+        else:
+            self.resid = None
+        self._taps = _TapCache()
+
+    def forward_safe(self, x):
+        """Arbitrary H, W (reference: dwoconv1d.py:154-187); handled natively."""
+        return self.forward(x)
+
+    def forward(self, x):
+        return _DepthwiseOrientedConv1d.apply(
+            x, self.weight, self.theta, self.bias, self, self.nhwc, self.resid
+        )

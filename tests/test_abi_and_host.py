@@ -1,0 +1,116 @@
+"""CPU-only checks: the C-ABI library loads and exports every symbol the header declares,
+argument validation returns the documented status codes before any GPU work, the host tap
+table equals the oracle's, and the operator module keeps the reference's contract
+(models/dwoconv1d/dwoconv1d.py:92-152)."""
+import ctypes
+import math
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+from oriented1d_amd import _lib
+from oriented1d_amd import dwoconv1d as op
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = _lib.load()
+    header = open(os.path.join(ROOT, "include", "dwoconv1d_hip.h")).read()
+    declared = set(re.findall(r"\b(dwo_[a-z0-9_]+)\s*\(", header))
+    assert declared, "no declarations parsed"
+    for name in sorted(declared):
+        assert hasattr(lib, name), "missing export " + name
+    assert declared == set(_lib.SIGNATURES), "ctypes table out of step with the header"
+    assert lib.dwo_version() >= 100
+
+
+def test_argument_validation_status_codes():
+    lib = _lib.load()
+    one = ctypes.c_void_p(16)  # never dereferenced: validation fails first
+
+    def fprop(N=1, C=1, H=4, W=4, K=7, stride=1, dtype=0, layout=0, x=one):
+        return lib.dwo_fprop(x, one, None, one, one, N, C, H, W, K, stride, dtype, layout, None)
+
+    assert fprop(x=None) == -1
+    assert fprop(N=0) == -2 and fprop(H=0) == -2
+    assert fprop(N=1 << 16, C=1 << 10, H=1 << 4, W=1 << 4) == -2  # >= 2^31 elements
+    assert fprop(K=8) == -3 and fprop(K=65) == -3 and fprop(K=0) == -3
+    assert fprop(stride=3) == -4
+    assert fprop(dtype=7) == -5
+    assert fprop(layout=2) == -6
+    assert lib.dwo_dgrad(None, one, one, one, 1, 1, 4, 4, 7, 1, 0, 0, None) == -1
+    need = lib.dwo_wgrad_scratch_bytes(2, 8, 8, 8, 7, 1, 0, 0)
+    assert need > 0
+    assert lib.dwo_wgrad(one, one, one, one, None, one, need - 1, 2, 8, 8, 8, 7, 1, 0, 0,
+                         None) == -7
+    assert lib.dwo_wgrad_scratch_bytes(2, 8, 8, 8, 8, 1, 0, 0) == 0
+    for code in (0, -1, -2, -3, -4, -5, -6, -7, -8):
+        assert lib.dwo_status_string(code)
+    assert lib.dwo_taps_bytes(8, 30) == 0
+    with pytest.raises(RuntimeError, match="stride must be"):
+        _lib.check(-4, "x")
+
+
+@pytest.mark.parametrize("K", [7, 13, 15, 27, 31, 63])
+def test_host_tap_table_equals_oracle(oracle, K):
+    rng = np.random.default_rng(K)
+    theta = np.concatenate([np.arange(8) * np.float32(math.pi / 8),
+                            [np.float32(math.pi * ((n / 8 + 0.5) % 1)) for n in range(8)],
+                            rng.uniform(-math.pi, 2 * math.pi, 48)]).astype(np.float32)
+    C = len(theta)
+    blob = op.build_taps(torch.from_numpy(theta), C, K)
+    dh, dw = op.taps_to_numpy(blob, C, K)
+    odh, odw = oracle.taps(theta, K)
+    assert (dh == odh).all() and (dw == odw).all()
+
+
+def test_module_contract():
+    C, K = 16, 31
+    angles = [math.pi * (c % 8) / 8 for c in range(C)]
+    m = op.DepthwiseOrientedConv1d(C, C, K, groups=C, padding=K // 2, angle=angles, resid=True)
+    assert isinstance(m, torch.nn.Conv2d)
+    assert list(m.state_dict().keys()) == ["weight", "bias", "theta"]
+    assert tuple(m.weight.shape) == (C, 1, 1, K) and tuple(m.bias.shape) == (C,)
+    assert tuple(m.theta.shape) == (C,) and m.theta.dtype == torch.float32
+    assert m.stride == (1, 1) and m.kernel_size == (1, K) and m.nhwc is False
+    assert tuple(m.resid.shape) == (C, 1, 1, K) and m.resid.sum() == C
+    assert m.resid[:, 0, 0, K // 2].eq(1).all()
+    # scalar angle -> [C,1] (dwoconv1d.py:128-129); no resid -> attribute is None
+    m2 = op.DepthwiseOrientedConv1d(C, C, 7, groups=C, angle=0.5, bias=False, nhwc=True, stride=2)
+    assert tuple(m2.theta.shape) == (C, 1) and m2.resid is None and m2.bias is None
+    assert op._DepthwiseOrientedConv1d.__name__ == "_DepthwiseOrientedConv1d"
+    with pytest.raises(AssertionError):
+        op.DepthwiseOrientedConv1d(C, C, 8, groups=C)  # even kernel
+    with pytest.raises(AssertionError):
+        op.DepthwiseOrientedConv1d(C, C, 7, groups=1)  # not depthwise
+    # reference check order: device first (kernels.cu:11-13)
+    with pytest.raises(RuntimeError, match="must be a CUDA tensor"):
+        m(torch.zeros(1, C, 8, 8))
+    import dwoconv1d as alias
+    assert alias.DepthwiseOrientedConv1d is op.DepthwiseOrientedConv1d
+
+
+def test_five_function_tuple_shape():
+    t = op.oriented_dwconv1d_get_module_from_params("float", 31, 1, 15, Sb=1)
+    assert len(t) == 5 and all(callable(f) for f in t)
+    x = torch.arange(24.).reshape(1, 2, 3, 4)
+    assert torch.equal(t[3](t[4](x)), x)
+
+
+def test_oracle_reproduces_golden_fixture(oracle):
+    import sys
+    sys.path.insert(0, os.path.join(ROOT, "tests", "golden"))
+    from make_golden import config1_inputs
+
+    g = np.load(os.path.join(ROOT, "tests", "golden", "config1_samples.npz"))
+    x, w, dy, theta = config1_inputs()
+    assert abs(x.astype(np.float64).sum() - g["x_sum"]) < 1e-9
+    assert abs(w.astype(np.float64).sum() - g["w_sum"]) < 1e-12
+    y = oracle.fprop(x, w, theta, threads=4).reshape(-1)[g["idx"]]
+    np.testing.assert_array_equal(y, g["y"])
+    dw = oracle.wgrad(dy, x, theta, 31, threads=4).reshape(96, 31)
+    np.testing.assert_array_equal(dw, g["dw"])

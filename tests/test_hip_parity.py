@@ -1,0 +1,170 @@
+"""GPU parity: the HIP kernels, called through the C ABI, against the CPU oracle on the same
+seeded inputs.  Tolerances: fp32 1e-5 relative, bf16/fp16 1e-2 relative (tensor-level, see
+parity_util.rel_err); wgrad is judged against the double-accumulating oracle because the
+reference's own serial fp32 sum over N*P*Q terms is noisier than 1e-5."""
+import math
+import os
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+from parity_util import (TOL, assert_close, canonical_theta, dev, grouped_theta, host, rel_err,
+                         rounded)
+
+pytestmark = pytest.mark.gpu
+
+from oriented1d_amd import dwoconv1d as op  # noqa: E402
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+DTYPES = [torch.float32, torch.bfloat16, torch.float16]
+
+
+def _case(oracle, N, C, H, W, K, stride, dtype, nhwc, theta, seed, bias=True, threads=8):
+    """Runs fprop, dgrad, wgrad(+db) through the C ABI and checks each against the oracle."""
+    rng = np.random.default_rng(seed)
+    x = rounded(rng.standard_normal((N, C, H, W)).astype(np.float32), dtype)
+    w = (rng.standard_normal((C, 1, 1, K)) * 0.02).astype(np.float32)
+    b = rng.standard_normal(C).astype(np.float32) if bias else None
+    P, Q = -(-H // stride), -(-W // stride)
+    dy = rounded(rng.standard_normal((N, C, P, Q)).astype(np.float32), dtype)
+    tag = "N%d C%d %dx%d K%d s%d %s %s" % (N, C, H, W, K, stride, dtype, "nhwc" if nhwc else "nchw")
+    print("case", tag, "seed", seed, flush=True)
+
+    def lay(a):
+        return np.ascontiguousarray(a.transpose(0, 2, 3, 1)) if nhwc else a
+
+    def unlay(a):
+        return a.transpose(0, 3, 1, 2) if nhwc else a
+
+    taps = op.build_taps(torch.from_numpy(theta), C, K).cuda()
+    xd, dyd, wd = dev(lay(x), dtype), dev(lay(dy), dtype), dev(w, torch.float32)
+    bd = dev(b, torch.float32) if bias else None
+
+    y = unlay(host(op.fprop(xd, wd, taps, stride, bias=bd, nhwc=nhwc)))
+    y_ref = oracle.fprop(x, w, theta, stride, threads=threads)
+    if bias:
+        y_ref = y_ref + b.astype(np.float64).reshape(1, -1, 1, 1)
+    assert_close(y, y_ref, dtype, tag + " fprop")
+
+    dx = unlay(host(op.dgrad(dyd, wd, taps, (H, W), stride, nhwc=nhwc)))
+    assert_close(dx, oracle.dgrad(dy, w, theta, stride, in_hw=(H, W), threads=threads), dtype,
+                 tag + " dgrad")
+
+    dw, db = op.wgrad(dyd, xd, taps, K, stride, nhwc=nhwc, with_bias=True)
+    # dw/db are fp32 sums of exact products of the (already rounded) inputs: fp32 tolerance
+    assert_close(host(dw), oracle.wgrad(dy, x, theta, K, stride, threads=threads), torch.float32,
+                 tag + " wgrad")
+    assert_close(host(db), oracle.bgrad(dy), torch.float32, tag + " bgrad")
+    torch.cuda.synchronize()
+
+
+def test_config1_cpu_runnable_case_and_golden(oracle):
+    """N=2, C=96, 56x56, K=31, theta=(c mod 8)*22.5deg, seed 0, fp32: full-tensor parity with
+    the oracle and with the committed golden samples."""
+    sys.path.insert(0, os.path.join(ROOT, "tests", "golden"))
+    from make_golden import config1_inputs
+
+    x, w, dy, theta = config1_inputs()
+    g = np.load(os.path.join(ROOT, "tests", "golden", "config1_samples.npz"))
+    taps = op.build_taps(torch.from_numpy(theta), 96, 31).cuda()
+    xd, wd, dyd = dev(x, torch.float32), dev(w, torch.float32), dev(dy, torch.float32)
+    y = host(op.fprop(xd, wd, taps))
+    assert_close(y, oracle.fprop(x, w, theta, threads=8), torch.float32, "config1 fprop")
+    assert_close(y.reshape(-1)[g["idx"]], g["y"], torch.float32, "config1 fprop golden")
+    dx = host(op.dgrad(dyd, wd, taps, (56, 56)))
+    assert_close(dx.reshape(-1)[g["idx"]], g["dx"], torch.float32, "config1 dgrad golden")
+    dw, _ = op.wgrad(dyd, xd, taps, 31)
+    assert_close(host(dw).reshape(96, 31), g["dw"], torch.float32, "config1 wgrad golden")
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=["f32", "bf16", "f16"])
+@pytest.mark.parametrize("nhwc", [False, True], ids=["nchw", "nhwc"])
+@pytest.mark.parametrize("C,HW", [(96, 56), (192, 28), (384, 14), (768, 7)])
+def test_stage_shapes_k31(oracle, C, HW, nhwc, dtype):
+    """ConvNeXt-T stage shapes (batch reduced to 4 so the oracle takes seconds)."""
+    _case(oracle, 4, C, HW, HW, 31, 1, dtype, nhwc, canonical_theta(C), seed=C + HW)
+
+
+@pytest.mark.parametrize("nhwc", [False, True], ids=["nchw", "nhwc"])
+@pytest.mark.parametrize("K", [7, 13, 15, 27, 31])
+def test_kernel_sizes_grouped_theta(oracle, K, nhwc):
+    """Cropped backbone kernel sizes; contiguous-group angles with the +90deg layer offset."""
+    _case(oracle, 2, 72, 20, 24, K, 1, torch.float32, nhwc, grouped_theta(72, 0.5), seed=K)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("nhwc", [False, True], ids=["nchw", "nhwc"])
+@pytest.mark.parametrize("stride,H,W,K", [(2, 32, 32, 31), (2, 24, 40, 15), (2, 15, 21, 15),
+                                          (4, 32, 24, 7), (2, 7, 9, 31)])
+def test_strided_and_odd_extents(oracle, stride, H, W, K, nhwc, dtype):
+    """Stem-like strided cases, including extents not divisible by the stride
+    (P = ceil(H/stride): the arbitrary-size semantics of dwoconv1d.py:154-187)."""
+    _case(oracle, 2, 64, H, W, K, stride, dtype, nhwc, grouped_theta(64), seed=H * W + K)
+
+
+@pytest.mark.parametrize("nhwc", [False, True], ids=["nchw", "nhwc"])
+def test_random_angles_ragged_shapes(oracle, nhwc):
+    rng = np.random.default_rng(77)
+    for (N, C, H, W, K) in [(1, 1, 1, 1, 31), (3, 5, 1, 9, 7), (2, 67, 9, 1, 15), (1, 130, 33, 17, 31),
+                            (2, 9, 61, 70, 31), (1, 3, 130, 140, 31)]:
+        theta = rng.uniform(-math.pi, 2 * math.pi, C).astype(np.float32)
+        _case(oracle, N, C, H, W, K, 1, torch.float32, nhwc, theta, seed=N * C + H)
+
+
+def test_wgrad_is_deterministic():
+    C, K = 96, 31
+    g = torch.Generator(device="cuda").manual_seed(5)
+    x = torch.randn(16, C, 56, 56, device="cuda", generator=g)
+    dy = torch.randn(16, C, 56, 56, device="cuda", generator=g)
+    taps = op.build_taps(torch.from_numpy(canonical_theta(C)), C, K).cuda()
+    a, adb = op.wgrad(dy, x, taps, K, with_bias=True)
+    b, bdb = op.wgrad(dy, x, taps, K, with_bias=True)
+    assert torch.equal(a, b) and torch.equal(adb, bdb)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("C,HW", [(96, 56), (192, 28), (384, 14), (768, 7)])
+def test_full_size_properties(oracle, C, HW, dtype):
+    """Batch-64 stage shapes: size-independent properties on the full tensors
+    (adjoint identities, linearity in x) plus oracle parity on two whole images."""
+    N, K = 64, 31
+    theta = canonical_theta(C)
+    g = torch.Generator(device="cuda").manual_seed(C)
+    x = torch.randn(N, C, HW, HW, device="cuda", generator=g).to(dtype)
+    dy = torch.randn(N, C, HW, HW, device="cuda", generator=g).to(dtype)
+    w = torch.randn(C, 1, 1, K, device="cuda", generator=g) * 0.02
+    taps = op.build_taps(torch.from_numpy(theta), C, K).cuda()
+    y = op.fprop(x, w, taps)
+    dx = op.dgrad(dy, w, taps, (HW, HW))
+    dw, db = op.wgrad(dy, x, taps, K, with_bias=True)
+    torch.cuda.synchronize()
+    # <y,dy> = <x,dx> = <w,dw>; terms are O(1) random so compare against sqrt(#terms) scale
+    a = (y.double() * dy.double()).sum().item()
+    b = (x.double() * dx.double()).sum().item()
+    c = (w.double() * dw.double()).sum().item()
+    scale = math.sqrt((y.double() ** 2).sum().item() * (dy.double() ** 2).sum().item())
+    tol = TOL[dtype]
+    assert abs(a - c) <= tol * scale and abs(a - b) <= tol * scale, (a, b, c, scale)
+    assert_close(host(db), host(dy.double().sum((0, 2, 3))), torch.float32, "db")
+    # linearity: fprop(2x) = 2 fprop(x) exactly (power-of-two scaling commutes with rounding)
+    assert torch.equal(op.fprop(x * 2, w, taps), y * 2)
+    # two whole images against the oracle
+    xs, dys = host(x[5:7]), host(dy[5:7])
+    assert_close(host(y[5:7]), oracle.fprop(xs, host(w), theta, threads=8), dtype, "fprop n=5,6")
+    assert_close(host(dx[5:7]), oracle.dgrad(dys, host(w), theta, threads=8), dtype, "dgrad n=5,6")
+
+
+def test_full_size_wgrad_against_oracle(oracle):
+    """wgrad at the full batch-64 reduction length for the two smallest stage shapes
+    (the oracle needs the whole batch; these finish in seconds on the host)."""
+    for C, HW in [(768, 7), (384, 14)]:
+        theta = canonical_theta(C)
+        rng = np.random.default_rng(C)
+        x = rng.standard_normal((64, C, HW, HW)).astype(np.float32)
+        dy = rng.standard_normal((64, C, HW, HW)).astype(np.float32)
+        taps = op.build_taps(torch.from_numpy(theta), C, 31).cuda()
+        dw, _ = op.wgrad(dev(dy, torch.float32), dev(x, torch.float32), taps, 31)
+        assert_close(host(dw), oracle.wgrad(dy, x, theta, 31, threads=8), torch.float32,
+                     "wgrad C%d %d^2" % (C, HW))
