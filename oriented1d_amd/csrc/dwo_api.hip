@@ -1,10 +1,12 @@
 // C ABI of libdwoconv1d_hip.so: argument validation, host-side tap table, kernel selection
 // and launch.  No device allocation, no retained pointers, no global mutable state.
 #include <math.h>
+#include <stdlib.h>
 #include <string.h>
 
 #include "dwo_common.h"
 #include "dwo_generic.h"
+#include "dwo_static.h"
 
 using namespace dwo;
 
@@ -55,9 +57,47 @@ WgradSplit wgrad_generic_split(const ConvDims &d, int layout) {
     return s;
 }
 
+// Images per workgroup for the LDS-staged plane kernels: about three workgroups per CU,
+// a whole number of staged batches each.
+int planes_per_group(int N, int C, int PB) {
+    static const int target = getenv("DWO_TARGET_WGS") ? atoi(getenv("DWO_TARGET_WGS")) : 768;
+    long g = ((long)N * C + target - 1) / target;
+    g = (g + PB - 1) / PB * PB;
+    if (g > N) g = (N + PB - 1) / PB * PB;
+    if (g < PB) g = PB;
+    return (int)g;
+}
+
+template <int OP, typename T, int K, int H, int W>
+int launch_plane(const void *src, const float *w, const float *bias, const void *taps, void *dst,
+                 const ConvDims &d, hipStream_t st) {
+    const int G = planes_per_group(d.N, d.C, Tile<H, W>::PB);
+    const int groups = (d.N + G - 1) / G;
+    plane_kernel<OP, T, K, H, W>
+        <<<dim3(d.C * groups), dim3(Tile<H, W>::NT), plane_kernel_lds_bytes<K, H, W>(), st>>>(
+            (const T *)src, w, bias, taps, (T *)dst, d.N, d.C, G);
+    return launch_status();
+}
+
+// NCHW, stride 1, compile-time plane extents: returns -100 when no such kernel is built.
+template <int OP, typename T>
+int try_plane(const void *src, const float *w, const float *bias, const void *taps, void *dst,
+              const ConvDims &d, int layout, hipStream_t st) {
+    if (layout != DWO_NCHW || d.stride != 1 || d.K != 31 || d.H != d.W) return -100;
+    switch (d.H) {
+        case 56: return launch_plane<OP, T, 31, 56, 56>(src, w, bias, taps, dst, d, st);
+        case 28: return launch_plane<OP, T, 31, 28, 28>(src, w, bias, taps, dst, d, st);
+        case 14: return launch_plane<OP, T, 31, 14, 14>(src, w, bias, taps, dst, d, st);
+        case 7: return launch_plane<OP, T, 31, 7, 7>(src, w, bias, taps, dst, d, st);
+        default: return -100;
+    }
+}
+
 template <typename T>
 int fprop_t(const void *x, const float *w, const float *bias, const void *taps, void *y,
             const ConvDims &d, int layout, hipStream_t st) {
+    const int fast = try_plane<OP_FPROP, T>(x, w, bias, taps, y, d, layout, st);
+    if (fast != -100) return fast;
     const int total = d.N * d.C * d.P * d.Q;
     const dim3 grid((total + 255) / 256), block(256);
     const int8_t *tp = taps_dhdw(taps);
@@ -73,6 +113,8 @@ int fprop_t(const void *x, const float *w, const float *bias, const void *taps, 
 template <typename T>
 int dgrad_t(const void *dy, const float *w, const void *taps, void *dx, const ConvDims &d,
             int layout, hipStream_t st) {
+    const int fast = try_plane<OP_DGRAD, T>(dy, w, nullptr, taps, dx, d, layout, st);
+    if (fast != -100) return fast;
     const int total = d.N * d.C * d.H * d.W;
     const dim3 grid((total + 255) / 256), block(256);
     const int8_t *tp = taps_dhdw(taps);
@@ -156,7 +198,15 @@ int dwo_build_taps(const float *theta_host, int C, int K, void *taps_host) {
             dhdw[((size_t)c * K + s) * 2 + 0] = (int8_t)(int)fh;
             dhdw[((size_t)c * K + s) * 2 + 1] = (int8_t)(int)fw;
         }
+        // canonical orientation: all K taps equal one of the eight compile-time patterns
         cls[c] = -1;
+        for (int o = 0; o < 8 && cls[c] < 0; o++) {
+            bool same = true;
+            for (int s = 0; s < K && same; s++)
+                same = dhdw[((size_t)c * K + s) * 2] == canon_dh(o, K, s) &&
+                       dhdw[((size_t)c * K + s) * 2 + 1] == canon_dw(o, K, s);
+            if (same) cls[c] = o;
+        }
     }
     return DWO_OK;
 }

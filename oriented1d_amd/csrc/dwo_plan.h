@@ -1,0 +1,151 @@
+// Compile-time description of the eight canonical orientations (k * 22.5 degrees).
+//
+// For a canonical orientation the tap offsets are known when the kernel is compiled, so the
+// K-tap gather is emitted as straight-line code: every LDS read has an immediate offset from
+// one per-lane base address, every FMA names its weight register directly, and a lane that
+// computes L neighbouring outputs along the line's step direction reads each LDS value once
+// and feeds it to every output that needs it (a register sliding window).
+//
+// Step direction e per orientation class:
+//   H  (0, 22.5, 157.5 deg)  e = (0, +1)   L outputs side by side in a row
+//   V  (67.5, 90, 112.5 deg) e = (+1, 0)   L outputs stacked in a column
+//   D  (45 deg)              e = (-1, +1)  L outputs up the anti-diagonal
+//   D  (135 deg)             e = (+1, +1)  L outputs down the diagonal
+// The "plan" lists, for an item whose first output sits at the origin, every distinct source
+// position (sh, sw) = tap + l*e, and for each which tap feeds which of the L outputs.
+#pragma once
+
+#include <stdint.h>
+
+#include <utility>
+
+#include "dwo_canon_taps.h"
+
+namespace dwo {
+
+enum { CLS_H = 0, CLS_V = 1, CLS_D = 2 };
+
+constexpr int orient_class(int o) {
+    return (o == 0 || o == 1 || o == 7) ? CLS_H : ((o == 2 || o == 6) ? CLS_D : CLS_V);
+}
+constexpr int step_h(int o) { return orient_class(o) == CLS_H ? 0 : (o == 2 ? -1 : 1); }
+constexpr int step_w(int o) { return orient_class(o) == CLS_V ? 0 : 1; }
+
+// taps of kernel size K are the central K entries of the size-63 rows
+constexpr int canon_dh(int o, int K, int s) { return kCanon.dh[o][s + (kCanonK - K) / 2]; }
+constexpr int canon_dw(int o, int K, int s) { return kCanon.dw[o][s + (kCanonK - K) / 2]; }
+
+constexpr int kMaxSrc = 320;
+constexpr int kMaxL = 8;
+
+struct Plan {
+    int nsrc = 0;                      // distinct source positions per item
+    int ndistinct = 0;                 // distinct tap offsets (duplicates folded)
+    int16_t sh[kMaxSrc] = {};          // source position relative to the item origin
+    int16_t sw[kMaxSrc] = {};
+    int8_t user[kMaxSrc][kMaxL] = {};  // representative tap feeding output l, or -1
+    int8_t rep[64] = {};               // rep[s]: first tap with the same offset as tap s,
+                                       // -1 for a tap that cannot reach the plane
+    int hmin = 0, hmax = 0, wmin = 0, wmax = 0;  // bounding box of the source positions
+};
+
+// Taps that can never land inside an H x W plane (|dh| >= H or |dw| >= W) are dropped: they
+// only ever read the zero halo.
+constexpr Plan make_plan(int o, int K, int L, int H, int W) {
+    Plan p{};
+    const int eh = step_h(o), ew = step_w(o);
+    constexpr int G = 48, GS = 2 * G + 1;
+    int8_t grid[GS][GS] = {};
+    for (int i = 0; i < GS; i++)
+        for (int j = 0; j < GS; j++) grid[i][j] = -1;
+    for (int s = 0; s < K; s++) {
+        const int dh = canon_dh(o, K, s), dw = canon_dw(o, K, s);
+        p.rep[s] = -1;
+        if (dh >= H || dh <= -H || dw >= W || dw <= -W) continue;
+        if (grid[dh + G][dw + G] < 0) {
+            grid[dh + G][dw + G] = (int8_t)s;
+            p.ndistinct++;
+        }
+        p.rep[s] = grid[dh + G][dw + G];
+        for (int l = 0; l < L; l++) {
+            const int h = dh + l * eh, w = dw + l * ew;
+            if (h < p.hmin) p.hmin = h;
+            if (h > p.hmax) p.hmax = h;
+            if (w < p.wmin) p.wmin = w;
+            if (w > p.wmax) p.wmax = w;
+        }
+    }
+    for (int h = p.hmin; h <= p.hmax; h++)
+        for (int w = p.wmin; w <= p.wmax; w++) {
+            bool any = false;
+            int8_t u[kMaxL] = {};
+            for (int l = 0; l < kMaxL; l++) u[l] = -1;
+            for (int l = 0; l < L; l++) {
+                const int th = h - l * eh + G, tw = w - l * ew + G;
+                if (th >= 0 && th < GS && tw >= 0 && tw < GS && grid[th][tw] >= 0) {
+                    u[l] = grid[th][tw];
+                    any = true;
+                }
+            }
+            if (any) {
+                p.sh[p.nsrc] = (int16_t)h;
+                p.sw[p.nsrc] = (int16_t)w;
+                for (int l = 0; l < kMaxL; l++) p.user[p.nsrc][l] = u[l];
+                p.nsrc++;
+            }
+        }
+    return p;
+}
+
+constexpr int round_up(int v, int m) { return (v + m - 1) / m * m; }
+constexpr int cmax(int a, int b) { return a > b ? a : b; }
+
+// Smallest r >= need with (mult * r - target) divisible by 32, or need rounded to odd when
+// no such r exists within one period.  Used to pick LDS row strides for which the flattened
+// item -> address map is linear modulo the 32 banks.
+constexpr int bank_stride(int need, int mult, int target) {
+    for (int r = need; r < need + 32; r++)
+        if ((mult * r - target) % 32 == 0) return r;
+    return need | 1;
+}
+
+// LDS geometry of one (orientation, K, L, H, W) variant.  All sizes in floats.
+template <int O, int K, int L, int H, int W>
+struct Geo {
+    static constexpr int CLS = orient_class(O);
+    static constexpr int EH = step_h(O), EW = step_w(O);
+    static constexpr Plan plan = make_plan(O, K, L, H, W);
+
+    static constexpr int LR = CLS == CLS_H ? 1 : L;              // rows per row-block
+    static constexpr int RB = (H + LR - 1) / LR;                 // row-blocks per plane
+    static constexpr int IPR = CLS == CLS_H ? W / L              // items per row-block
+                               : (CLS == CLS_V ? W : round_up(W + L - 1, 8));
+    static constexpr int IPP = RB * IPR;                         // items per plane
+    static constexpr int P0 = (CLS == CLS_D && EH < 0) ? L - 1 : 0;  // origin row in the block
+    static constexpr int PT = cmax(0, -(P0 + plan.hmin));        // zero rows above the plane
+    static constexpr int ROWS = cmax(H + PT, (RB - 1) * LR + P0 + plan.hmax + PT + 1);
+
+    // columns
+    static constexpr int Q0 = CLS == CLS_D ? L - 1 : 0;  // item j's origin column is j - Q0
+    static constexpr int PL =
+        CLS == CLS_H ? round_up(cmax(0, -plan.wmin), L) : round_up(cmax(0, Q0 - plan.wmin), 4);
+    // H class: a padded row is split into L sub-rows, column u lives in sub-row u % L at u / L
+    static constexpr int SUB = (PL + W - 1 + cmax(0, plan.wmax)) / L + 1;
+    static constexpr int WIDTH =
+        CLS == CLS_H ? L * SUB
+                     : (CLS == CLS_V ? PL + W + cmax(0, plan.wmax)
+                                     : PL + cmax(W, IPR - Q0) + cmax(0, plan.wmax));
+    static constexpr int RS = bank_stride(WIDTH, LR, IPR);
+    static constexpr int PLANE = ROWS * RS;  // floats per staged plane
+
+    // LDS offset of column u (already including PL) within a row
+    static constexpr int col(int u) { return CLS == CLS_H ? (u % L) * SUB + u / L : u; }
+    // immediate offset of source (sh, sw) from the item base  rb*LR*RS + j
+    static constexpr int imm(int sh, int sw) {
+        return (sh + P0 + PT) * RS + (CLS == CLS_H ? col(sw + PL) : sw + PL - Q0);
+    }
+    // LDS index of interior element (r, w) of the plane
+    static constexpr int interior_row(int r) { return (r + PT) * RS; }
+};
+
+}  // namespace dwo
