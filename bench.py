@@ -194,7 +194,7 @@ def main():
         from oracle import dwo_oracle as oracle
 
         rng = np.random.default_rng(0)
-        n_cpu = 4  # bounded sample: 4 of the 64 images at every stage shape, all three ops
+        n_cpu = BATCH  # the whole step once: every stage shape at batch 64, all three ops
         cpu_bytes, cpu_s = 0, 0.0
         for C, HW in STAGES:
             th = theta_for(C)
@@ -210,8 +210,9 @@ def main():
                              for o in ("fprop", "dgrad", "wgrad"))
         cpu = {"value": round(cpu_bytes / cpu_s / 1e9, 4), "unit": "GB/s", "cores": 1,
                "kind": "port",
-               "sample": "fp32 fprop+dgrad+wgrad, 4 of 64 images at each of the four stage "
-                         "shapes, single thread, reference loop order (%.1f s)" % cpu_s,
+               "sample": "one whole step: fp32 fprop+dgrad+wgrad at each of the four stage shapes, "
+                         "batch 64, single thread, reference loop order and fp32 accumulation "
+                         "(%.1f s)" % cpu_s,
                "host_cpus": os.cpu_count()}
 
     out = {

@@ -3,7 +3,8 @@ import ctypes
 import os
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(HERE, "libdwoconv1d_hip.so")
+# DWOCONV1D_LIB overrides the library location (e.g. an instrumented build)
+LIB_PATH = os.environ.get("DWOCONV1D_LIB") or os.path.join(HERE, "libdwoconv1d_hip.so")
 
 F32, BF16, F16 = 0, 1, 2
 NCHW, NHWC = 0, 1

@@ -16,6 +16,10 @@ HIPCC_FLAGS = [
     "-shared",
     # packed fp32 VALU forms are disabled for every device function in this library
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # LDS reads keep their own 16-bit immediate offsets: merging them into ds_read2 forms
+    # (8-bit offsets) costs one address add per pair in the unrolled tap gathers
+    "-Xclang", "-target-feature", "-Xclang", "-load-store-opt",
+    "-mllvm", "-amdgpu-load-store-vectorizer=0",
     "-Wno-unused-command-line-argument",
 ]
 
@@ -27,21 +31,43 @@ def hipcc():
     return exe
 
 
-def build(verbose=False):
-    """Compile csrc/dwo_api.hip (which includes every kernel header) into the package dir."""
-    cmd = [hipcc()] + HIPCC_FLAGS + [
-        "-I" + os.path.join(ROOT, "include"), "-I" + CSRC,
-        os.path.join(CSRC, "dwo_api.hip"), "-o", LIB + ".tmp",
-    ]
+PLANE_SHAPES = [(31, 56, 56), (31, 28, 28), (31, 14, 14), (31, 7, 7)]  # = DWO_PLANE_SHAPES
+PLANE_TYPES = ["float", "bf16_t", "f16_t"]
+
+
+def _run(cmd, verbose):
     if verbose:
         print(" ".join(cmd), flush=True)
     proc = subprocess.run(cmd, capture_output=True, text=True)
     # the host pass reports that it does not know the packed-fp32 feature: harmless
-    err = "\n".join(l for l in proc.stderr.splitlines() if "packed-fp32-ops" not in l)
+    err = "\n".join(l for l in proc.stderr.splitlines() if "packed-fp32-ops" not in l and "load-store-opt" not in l)
     if proc.returncode != 0:
-        raise RuntimeError("hipcc failed:\n" + err)
+        raise RuntimeError("hipcc failed: %s\n%s" % (" ".join(cmd), err))
     if verbose and err.strip():
         print(err)
+
+
+def build(verbose=False, jobs=None):
+    """Compile csrc/dwo_api.hip and one csrc/dwo_inst.hip object per (element type, plane
+    extent) in parallel, then link libdwoconv1d_hip.so into the package directory."""
+    from concurrent.futures import ThreadPoolExecutor
+
+    objdir = os.path.join(HERE, "build")
+    os.makedirs(objdir, exist_ok=True)
+    common = [hipcc()] + [f for f in HIPCC_FLAGS if f != "-shared"] + [
+        "-I" + os.path.join(ROOT, "include"), "-I" + CSRC, "-c"]
+    units = [(os.path.join(CSRC, "dwo_api.hip"), os.path.join(objdir, "dwo_api.o"), [])]
+    for K, H, W in PLANE_SHAPES:
+        for t in PLANE_TYPES:
+            units.append((os.path.join(CSRC, "dwo_inst.hip"),
+                          os.path.join(objdir, "dwo_inst_%s_k%d_%dx%d.o" % (t, K, H, W)),
+                          ["-DDWO_INST_T=" + t, "-DDWO_INST_K=%d" % K, "-DDWO_INST_H=%d" % H,
+                           "-DDWO_INST_W=%d" % W]))
+    jobs = jobs or min(len(units), max(1, min(16, os.cpu_count() or 1)))
+    with ThreadPoolExecutor(jobs) as pool:
+        list(pool.map(lambda u: _run(common + u[2] + [u[0], "-o", u[1]], verbose), units))
+    _run([hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC"] + [u[1] for u in units] +
+         ["-o", LIB + ".tmp"], verbose)
     os.replace(LIB + ".tmp", LIB)
     return LIB
 

@@ -6,7 +6,7 @@
 
 #include "dwo_common.h"
 #include "dwo_generic.h"
-#include "dwo_static.h"
+#include "dwo_dispatch.h"
 
 using namespace dwo;
 
@@ -57,46 +57,54 @@ WgradSplit wgrad_generic_split(const ConvDims &d, int layout) {
     return s;
 }
 
-// Images per workgroup for the LDS-staged plane kernels: about three workgroups per CU,
-// a whole number of staged batches each.
-int planes_per_group(int N, int C, int PB) {
-    static const int target = getenv("DWO_TARGET_WGS") ? atoi(getenv("DWO_TARGET_WGS")) : 768;
-    long g = ((long)N * C + target - 1) / target;
-    g = (g + PB - 1) / PB * PB;
-    if (g > N) g = (N + PB - 1) / PB * PB;
-    if (g < PB) g = PB;
-    return (int)g;
+// Plane extents with LDS-staged kernels (NCHW, stride 1).  PB = planes staged per batch.
+int plane_batch(const ConvDims &d, int layout) {
+    if (layout != DWO_NCHW || d.stride != 1) return 0;
+#define DWO_MATCH(K_, H_, W_) \
+    if (d.K == K_ && d.H == H_ && d.W == W_) return Tile<H_, W_>::PB;
+    DWO_PLANE_SHAPES(DWO_MATCH)
+#undef DWO_MATCH
+    return 0;
 }
 
-template <int OP, typename T, int K, int H, int W>
-int launch_plane(const void *src, const float *w, const float *bias, const void *taps, void *dst,
-                 const ConvDims &d, hipStream_t st) {
-    const int G = planes_per_group(d.N, d.C, Tile<H, W>::PB);
-    const int groups = (d.N + G - 1) / G;
-    plane_kernel<OP, T, K, H, W>
-        <<<dim3(d.C * groups), dim3(Tile<H, W>::NT), plane_kernel_lds_bytes<K, H, W>(), st>>>(
-            (const T *)src, w, bias, taps, (T *)dst, d.N, d.C, G);
-    return launch_status();
+// returns -100 when no LDS-staged kernel covers the shape
+template <typename T>
+int try_plane_conv(int op, const void *src, const float *w, const float *bias, const void *taps,
+                   void *dst, const ConvDims &d, int layout, hipStream_t st) {
+    if (plane_batch(d, layout) == 0) return -100;
+#define DWO_MATCH(K_, H_, W_)                                                               \
+    if (d.K == K_ && d.H == H_ && d.W == W_)                                                \
+        return launch_plane_conv<T, K_, H_, W_>(op, src, w, bias, taps, dst, d.N, d.C, st);
+    DWO_PLANE_SHAPES(DWO_MATCH)
+#undef DWO_MATCH
+    return -100;
 }
 
-// NCHW, stride 1, compile-time plane extents: returns -100 when no such kernel is built.
-template <int OP, typename T>
-int try_plane(const void *src, const float *w, const float *bias, const void *taps, void *dst,
-              const ConvDims &d, int layout, hipStream_t st) {
-    if (layout != DWO_NCHW || d.stride != 1 || d.K != 31 || d.H != d.W) return -100;
-    switch (d.H) {
-        case 56: return launch_plane<OP, T, 31, 56, 56>(src, w, bias, taps, dst, d, st);
-        case 28: return launch_plane<OP, T, 31, 28, 28>(src, w, bias, taps, dst, d, st);
-        case 14: return launch_plane<OP, T, 31, 14, 14>(src, w, bias, taps, dst, d, st);
-        case 7: return launch_plane<OP, T, 31, 7, 7>(src, w, bias, taps, dst, d, st);
-        default: return -100;
-    }
+template <typename T>
+int try_plane_wgrad(const void *x, const void *dy, const void *taps, float *part, int *groups,
+                    const ConvDims &d, hipStream_t st) {
+#define DWO_MATCH(K_, H_, W_)                                                               \
+    if (d.K == K_ && d.H == H_ && d.W == W_)                                                \
+        return launch_plane_wgrad<T, K_, H_, W_>(x, dy, taps, part, d.N, d.C, groups, st);
+    DWO_PLANE_SHAPES(DWO_MATCH)
+#undef DWO_MATCH
+    return -100;
+}
+
+// wgrad partial-sum count per (channel, tap): an upper bound that sizes the scratch buffer
+// (the staged path picks its group count from the device's occupancy at launch, never more
+// than kMaxPlaneGroups nor than the number of staged batches).
+int wgrad_max_partials(const ConvDims &d, int layout) {
+    const int PB = plane_batch(d, layout);
+    if (PB == 0) return wgrad_generic_split(d, layout).G;
+    const int nbatch = (d.N + PB - 1) / PB;
+    return nbatch < kMaxPlaneGroups ? nbatch : kMaxPlaneGroups;
 }
 
 template <typename T>
 int fprop_t(const void *x, const float *w, const float *bias, const void *taps, void *y,
             const ConvDims &d, int layout, hipStream_t st) {
-    const int fast = try_plane<OP_FPROP, T>(x, w, bias, taps, y, d, layout, st);
+    const int fast = try_plane_conv<T>(OP_FPROP, x, w, bias, taps, y, d, layout, st);
     if (fast != -100) return fast;
     const int total = d.N * d.C * d.P * d.Q;
     const dim3 grid((total + 255) / 256), block(256);
@@ -113,7 +121,7 @@ int fprop_t(const void *x, const float *w, const float *bias, const void *taps, 
 template <typename T>
 int dgrad_t(const void *dy, const float *w, const void *taps, void *dx, const ConvDims &d,
             int layout, hipStream_t st) {
-    const int fast = try_plane<OP_DGRAD, T>(dy, w, nullptr, taps, dx, d, layout, st);
+    const int fast = try_plane_conv<T>(OP_DGRAD, dy, w, nullptr, taps, dx, d, layout, st);
     if (fast != -100) return fast;
     const int total = d.N * d.C * d.H * d.W;
     const dim3 grid((total + 255) / 256), block(256);
@@ -130,21 +138,27 @@ int dgrad_t(const void *dy, const float *w, const void *taps, void *dx, const Co
 template <typename T>
 int wgrad_t(const void *dy, const void *x, const void *taps, float *dw, float *db, void *scratch,
             const ConvDims &d, int layout, hipStream_t st) {
-    const WgradSplit s = wgrad_generic_split(d, layout);
-    const dim3 grid(s.blocks_x, s.G), block(256);
-    const int8_t *tp = taps_dhdw(taps);
     float *part = (float *)scratch;
-    if (layout == DWO_NCHW)
-        wgrad_generic_kernel<T, DWO_NCHW><<<grid, block, 0, st>>>((const T *)dy, (const T *)x, tp,
-                                                                  part, d, s.G, s.per_slice);
-    else
-        wgrad_generic_kernel<T, DWO_NHWC><<<grid, block, 0, st>>>((const T *)dy, (const T *)x, tp,
-                                                                  part, d, s.G, s.per_slice);
-    int rc = launch_status();
+    int rc, NG = 0;
+    if (plane_batch(d, layout) != 0) {
+        rc = try_plane_wgrad<T>(x, dy, taps, part, &NG, d, st);
+    } else {
+        const WgradSplit s = wgrad_generic_split(d, layout);
+        NG = s.G;
+        const dim3 grid(s.blocks_x, s.G), block(256);
+        const int8_t *tp = taps_dhdw(taps);
+        if (layout == DWO_NCHW)
+            wgrad_generic_kernel<T, DWO_NCHW><<<grid, block, 0, st>>>(
+                (const T *)dy, (const T *)x, tp, part, d, s.G, s.per_slice);
+        else
+            wgrad_generic_kernel<T, DWO_NHWC><<<grid, block, 0, st>>>(
+                (const T *)dy, (const T *)x, tp, part, d, s.G, s.per_slice);
+        rc = launch_status();
+    }
     if (rc != DWO_OK) return rc;
     const int cells = d.C * (d.K + 1);
     wgrad_reduce_kernel<<<dim3((cells + 255) / 256), dim3(256), 0, st>>>(part, dw, db, d.C, d.K,
-                                                                        s.G);
+                                                                        NG);
     return launch_status();
 }
 
@@ -254,8 +268,7 @@ size_t dwo_wgrad_scratch_bytes(int N, int C, int H, int W, int K, int stride, in
                                int layout) {
     if (check_common(N, C, H, W, K, stride, dtype, layout) != DWO_OK) return 0;
     const ConvDims d = make_dims(N, C, H, W, K, stride);
-    const WgradSplit s = wgrad_generic_split(d, layout);
-    return (size_t)C * (K + 1) * s.G * sizeof(float);
+    return (size_t)C * (K + 1) * wgrad_max_partials(d, layout) * sizeof(float);
 }
 
 int dwo_wgrad(const void *dy, const void *x, const void *taps, float *dw, float *db,

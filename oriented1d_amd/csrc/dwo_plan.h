@@ -113,6 +113,7 @@ constexpr int bank_stride(int need, int mult, int target) {
 template <int O, int K, int L, int H, int W>
 struct Geo {
     static constexpr int CLS = orient_class(O);
+    static constexpr int L_ = L;
     static constexpr int EH = step_h(O), EW = step_w(O);
     static constexpr Plan plan = make_plan(O, K, L, H, W);
 
@@ -147,5 +148,37 @@ struct Geo {
     // LDS index of interior element (r, w) of the plane
     static constexpr int interior_row(int r) { return (r + PT) * RS; }
 };
+
+// Work decomposition per plane extent: outputs per lane (L) for each orientation class, planes
+// staged per batch (PB) and threads per workgroup (NT), chosen so that one batch yields close
+// to NT items for every class (items per plane: H class H*W/LH, V class ceil(H/LV)*W, D class
+// ceil(H/LD)*round_up(W+LD-1, 8)).
+template <int H, int W>
+struct Tile {
+    static constexpr int LH = W % 4 == 0 ? 4 : (W % 2 == 0 ? 2 : 1);
+    static constexpr int LV = LH, LD = LH;
+    static constexpr int PB = 1, NT = 256;
+};
+template <>
+struct Tile<56, 56> {  // 784 / 448 / 448 items per plane
+    static constexpr int LH = 4, LV = 7, LD = 8, PB = 1, NT = 448;
+};
+template <>
+struct Tile<28, 28> {  // 196 / 196 / 224
+    static constexpr int LH = 4, LV = 4, LD = 4, PB = 2, NT = 448;
+};
+template <>
+struct Tile<14, 14> {  // 98 / 98 / 112
+    static constexpr int LH = 2, LV = 2, LD = 2, PB = 4, NT = 448;
+};
+template <>
+struct Tile<7, 7> {  // 49 / 49 / 56
+    static constexpr int LH = 1, LV = 1, LD = 1, PB = 8, NT = 448;
+};
+template <int H, int W>
+constexpr int tile_L(int o) {
+    return orient_class(o) == CLS_H ? Tile<H, W>::LH
+                                    : (orient_class(o) == CLS_V ? Tile<H, W>::LV : Tile<H, W>::LD);
+}
 
 }  // namespace dwo

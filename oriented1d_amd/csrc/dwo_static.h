@@ -8,7 +8,17 @@
 // the table-driven body at the bottom (same staging, dynamic taps).
 #pragma once
 
+#include <stdlib.h>
+
+#ifndef DWO_WPE
+#define DWO_WPE 6
+#endif
+#ifndef DWO_WPE_WGRAD
+#define DWO_WPE_WGRAD 6
+#endif
+
 #include "dwo_common.h"
+#include "dwo_dispatch.h"
 #include "dwo_plan.h"
 
 namespace dwo {
@@ -22,24 +32,40 @@ __device__ __forceinline__ void static_for(F &&f) {
     static_for_impl(f, std::make_integer_sequence<int, N>{});
 }
 
-enum { OP_FPROP = 0, OP_DGRAD = 1 };
+
 
 // Four consecutive activations of type T as floats (one 16-byte or 8-byte global access).
+// Activations are touched exactly once per pass, so all global accesses are non-temporal:
+// outputs stream to HBM while the kernel runs instead of sitting dirty in L2 until the
+// end-of-kernel write-back, and inputs do not displace them.
 template <typename T>
 struct Vec4;
+// (native vector types: each load/store below is a single 16- or 8-byte memory instruction)
 template <>
 struct Vec4<float> {
-    float4 v;
-    __device__ __forceinline__ void load(const float *p) { v = *reinterpret_cast<const float4 *>(p); }
-    __device__ __forceinline__ void store(float *p) const { *reinterpret_cast<float4 *>(p) = v; }
-    __device__ __forceinline__ float get(int i) const { return i == 0 ? v.x : (i == 1 ? v.y : (i == 2 ? v.z : v.w)); }
-    __device__ __forceinline__ void set(float a, float b, float c, float d) { v = make_float4(a, b, c, d); }
+    typedef float f4 __attribute__((ext_vector_type(4)));
+    f4 v;
+    __device__ __forceinline__ void load(const float *p) {
+        v = __builtin_nontemporal_load(reinterpret_cast<const f4 *>(p));
+    }
+    __device__ __forceinline__ void store(float *p) const {
+        __builtin_nontemporal_store(v, reinterpret_cast<f4 *>(p));
+    }
+    __device__ __forceinline__ float get(int i) const { return v[i]; }
+    __device__ __forceinline__ void set(float a, float b, float c, float d) {
+        v[0] = a, v[1] = b, v[2] = c, v[3] = d;
+    }
 };
 template <>
 struct Vec4<bf16_t> {
-    uint2 v;
-    __device__ __forceinline__ void load(const bf16_t *p) { v = *reinterpret_cast<const uint2 *>(p); }
-    __device__ __forceinline__ void store(bf16_t *p) const { *reinterpret_cast<uint2 *>(p) = v; }
+    typedef uint32_t u2 __attribute__((ext_vector_type(2)));
+    u2 v;
+    __device__ __forceinline__ void load(const bf16_t *p) {
+        v = __builtin_nontemporal_load(reinterpret_cast<const u2 *>(p));
+    }
+    __device__ __forceinline__ void store(bf16_t *p) const {
+        __builtin_nontemporal_store(v, reinterpret_cast<u2 *>(p));
+    }
     __device__ __forceinline__ float get(int i) const {
         const uint32_t w = i < 2 ? v.x : v.y;
         return __uint_as_float((i & 1) ? (w & 0xffff0000u) : (w << 16));
@@ -53,45 +79,17 @@ template <>
 struct Vec4<f16_t> {
     typedef _Float16 h4 __attribute__((ext_vector_type(4)));
     h4 v;
-    __device__ __forceinline__ void load(const f16_t *p) { v = *reinterpret_cast<const h4 *>(p); }
-    __device__ __forceinline__ void store(f16_t *p) const { *reinterpret_cast<h4 *>(p) = v; }
+    __device__ __forceinline__ void load(const f16_t *p) {
+        v = __builtin_nontemporal_load(reinterpret_cast<const h4 *>(p));
+    }
+    __device__ __forceinline__ void store(f16_t *p) const {
+        __builtin_nontemporal_store(v, reinterpret_cast<h4 *>(p));
+    }
     __device__ __forceinline__ float get(int i) const { return (float)v[i]; }
     __device__ __forceinline__ void set(float a, float b, float c, float d) {
         v[0] = (_Float16)a, v[1] = (_Float16)b, v[2] = (_Float16)c, v[3] = (_Float16)d;
     }
 };
-
-// Work decomposition per plane extent: outputs per lane (L) for each orientation class, planes
-// staged per batch (PB) and threads per workgroup (NT), chosen so that one batch yields close
-// to NT items for every class (items per plane: H class H*W/LH, V class ceil(H/LV)*W, D class
-// ceil(H/LD)*round_up(W+LD-1, 8)).
-template <int H, int W>
-struct Tile {
-    static constexpr int LH = W % 4 == 0 ? 4 : (W % 2 == 0 ? 2 : 1);
-    static constexpr int LV = LH, LD = LH;
-    static constexpr int PB = 1, NT = 256;
-};
-template <>
-struct Tile<56, 56> {  // 784 / 448 / 448 items per plane
-    static constexpr int LH = 4, LV = 7, LD = 8, PB = 1, NT = 448;
-};
-template <>
-struct Tile<28, 28> {  // 196 / 196 / 224
-    static constexpr int LH = 4, LV = 4, LD = 4, PB = 2, NT = 448;
-};
-template <>
-struct Tile<14, 14> {  // 98 / 98 / 112
-    static constexpr int LH = 2, LV = 2, LD = 2, PB = 4, NT = 448;
-};
-template <>
-struct Tile<7, 7> {  // 49 / 49 / 56
-    static constexpr int LH = 1, LV = 1, LD = 1, PB = 8, NT = 448;
-};
-template <int H, int W>
-constexpr int tile_L(int o) {
-    return orient_class(o) == CLS_H ? Tile<H, W>::LH
-                                    : (orient_class(o) == CLS_V ? Tile<H, W>::LV : Tile<H, W>::LD);
-}
 
 // halo of the table-driven body: no live tap reaches further than this
 template <int K, int H, int W>
@@ -111,6 +109,18 @@ constexpr int plane_floats() {
     return max_plane_floats<K, H, W>(std::make_integer_sequence<int, 8>{});
 }
 
+// scalar non-temporal store (bf16_t is a struct: store its bits)
+__device__ __forceinline__ void st_out(float *p, float v) { __builtin_nontemporal_store(v, p); }
+#ifdef DWO_NT_SCALAR16
+__device__ __forceinline__ void st_out(f16_t *p, f16_t v) { __builtin_nontemporal_store(v, p); }
+__device__ __forceinline__ void st_out(bf16_t *p, bf16_t v) {
+    __builtin_nontemporal_store(v.bits, &p->bits);
+}
+#else
+__device__ __forceinline__ void st_out(f16_t *p, f16_t v) { *p = v; }
+__device__ __forceinline__ void st_out(bf16_t *p, bf16_t v) { *p = v; }
+#endif
+
 // VL consecutive activations of a plane held in registers between the global load and the LDS
 // write (VL = 4: one 16/8-byte access; VL = 1: planes whose size is not a multiple of four).
 template <typename T, int VL>
@@ -125,43 +135,115 @@ struct Chunk<T, 1> {
 };
 
 // Staging of PB planes (n, c), n = nb .. nb+PB-1, through registers into LDS.  `Map` gives the
-// LDS index of interior element (r, w) relative to the plane's LDS origin.
-template <typename T, int H, int W, int PB, int NT, int PLS, class Map>
+// LDS index of interior element (r, w) relative to the plane's LDS origin, PLS the LDS distance
+// between planes.  Global addresses are a uniform 64-bit base (plane (nb, c)) plus an unsigned
+// 32-bit per-lane element offset.  Loads do not depend on the channel's orientation, so the
+// kernels issue the first ones before they know which body will run.
+template <typename T, int H, int W, int PB, int NT>
 struct Stager {
     static constexpr int VL = (H * W) % 4 == 0 ? 4 : 1;
     static constexpr int FP = H * W / VL;              // chunks per plane
     static constexpr int PF = (PB * FP + NT - 1) / NT; // chunks per thread
     Chunk<T, VL> pre[PF];
 
-    __device__ __forceinline__ void prefetch(const T *__restrict__ src, int c, int C, int nb, int n1) {
+    // base = first plane of the batch; `nvalid` planes of the batch exist
+    __device__ __forceinline__ void prefetch(const T *__restrict__ base, unsigned plane_stride,
+                                             int nvalid) {
 #pragma unroll
         for (int k = 0; k < PF; k++) {
-            const int f = threadIdx.x + k * NT;
-            const int pl = f / FP, g = f % FP;
-            if (f < PB * FP && nb + pl < n1)
-                pre[k].load(src + ((size_t)(nb + pl) * C + c) * (H * W) + g * VL);
+            const unsigned f = threadIdx.x + k * NT;
+            const unsigned pl = f / FP, g = f % FP;
+            if (f < PB * FP && (int)pl < nvalid) pre[k].load(base + (pl * plane_stride + g * VL));
         }
     }
-    __device__ __forceinline__ void commit(float *lds, int nb, int n1) const {
+    template <class Map, int PLS>
+    __device__ __forceinline__ void commit(float *lds, int nvalid) const {
 #pragma unroll
         for (int k = 0; k < PF; k++) {
-            const int f = threadIdx.x + k * NT;
-            const int pl = f / FP, g = f % FP;
-            if (f < PB * FP && nb + pl < n1) {
+            const unsigned f = threadIdx.x + k * NT;
+            const unsigned pl = f / FP, g = f % FP;
+            if (f < PB * FP && (int)pl < nvalid) {
                 float *plane = lds + pl * PLS;
                 if constexpr (W % VL == 0) {
-                    const int r = g / (W / VL), w0 = (g % (W / VL)) * VL;
+                    const unsigned r = g / (W / VL), w0 = (g % (W / VL)) * VL;
+                    float *q = plane + Map::index(r, w0);
 #pragma unroll
-                    for (int e = 0; e < VL; e++) plane[Map::index(r, w0 + e)] = pre[k].get(e);
+                    for (int e = 0; e < VL; e++) q[Map::step(e)] = pre[k].get(e);
                 } else {
 #pragma unroll
                     for (int e = 0; e < VL; e++) {
-                        const int i = g * VL + e;
+                        const unsigned i = g * VL + e;
                         plane[Map::index(i / W, i % W)] = pre[k].get(e);
                     }
                 }
             }
         }
+    }
+};
+
+// Interior-element map of a canonical geometry.  step(e) is the LDS distance from element
+// (r, w0) to (r, w0 + e) when w0 is a multiple of four and the row is at least four wide.
+template <class G>
+struct GeoMap {
+    static __device__ __forceinline__ unsigned index(unsigned r, unsigned w) {
+        return G::interior_row(r) + G::col(w + G::PL);
+    }
+    static constexpr int step(int e) {
+        return G::CLS == CLS_H ? (G::L_ >= 4 ? (e % G::L_) * G::SUB + e / G::L_
+                                             : G::col(e + G::PL) - G::col(G::PL))
+                               : e;
+    }
+};
+
+// Wave priority from the fraction of the workgroup's images still to do.  The hardware issues
+// oldest-wave-first, so of the workgroups sharing a CU the youngest would otherwise starve, end
+// last and run its tail alone at low occupancy; raising the priority of whoever has most work
+// left keeps co-resident workgroups in step so that they finish together.
+__device__ __forceinline__ void set_progress_priority(int remaining, int total) {
+#ifndef DWO_NO_PRIO
+    const int level = (remaining * 4 - 1) / total;  // 3 .. 0
+    if (level >= 3)
+        __builtin_amdgcn_s_setprio(3);
+    else if (level == 2)
+        __builtin_amdgcn_s_setprio(2);
+    else if (level == 1)
+        __builtin_amdgcn_s_setprio(1);
+    else
+        __builtin_amdgcn_s_setprio(0);
+#endif
+}
+
+// Workgroup -> (channel, image group).  Hardware hands consecutive workgroup ids to the eight
+// XCDs round-robin and fills the CUs of an XCD in order, while orientation (hence cost) often
+// repeats with period 8 over the channels; rotating the task id inside every aligned block of
+// eight ids by (block + block/32) gives every XCD and every CU a mix of orientations.
+__device__ __forceinline__ void plane_task(int C, int groups, int &c, int &group) {
+    const int i = blockIdx.x, total = C * groups;
+    const int j = i >> 3;
+    int t = i;
+    if (j * 8 + 8 <= total) t = (j << 3) + ((i + j + (j >> 5)) & 7);
+    c = t % C;
+    group = t / C;
+}
+// Images [n0, n1) of group g: the ceil(N/PB) staged batches are split as evenly as possible.
+template <int PB>
+__device__ __forceinline__ void group_range(int N, int groups, int g, int &n0, int &n1) {
+    const int nbatch = (N + PB - 1) / PB;
+    n0 = (int)(((long)g * nbatch) / groups) * PB;
+    n1 = min((int)(((long)(g + 1) * nbatch) / groups) * PB, N);
+}
+
+// The two register sets of the fprop/dgrad pipeline; start() issues the loads of the first two
+// batches of images [n0, n1) of channel c.
+template <typename T, int H, int W>
+struct ConvStagers {
+    Stager<T, H, W, Tile<H, W>::PB, Tile<H, W>::NT> a, b;
+    __device__ __forceinline__ void start(const T *__restrict__ src, int c, int C, int n0, int n1) {
+        constexpr int PB = Tile<H, W>::PB;
+        const unsigned pstride = (unsigned)C * (H * W);
+        const T *sbase = src + (size_t)c * (H * W);
+        a.prefetch(sbase + (size_t)n0 * pstride, pstride, n1 - n0);
+        if (n0 + PB < n1) b.prefetch(sbase + (size_t)(n0 + PB) * pstride, pstride, n1 - n0 - PB);
     }
 };
 
@@ -171,17 +253,15 @@ struct Stager {
 template <int O, int OP, typename T, int K, int H, int W>
 __device__ __forceinline__ void run_canonical(const T *__restrict__ src, const float *__restrict__ wt,
                                               const float *__restrict__ bias, T *__restrict__ dst,
-                                              float *lds, int c, int C, int n0, int n1) {
+                                              float *lds, int c, int C, int n0, int n1,
+                                              ConvStagers<T, H, W> &sg) {
     constexpr int L = tile_L<H, W>(O);
     constexpr int PB = Tile<H, W>::PB, NT = Tile<H, W>::NT;
     using G = Geo<O, K, L, H, W>;
     constexpr int PLS = plane_floats<K, H, W>();  // LDS plane stride (same for all orientations)
-    struct Map {
-        static __device__ __forceinline__ int index(int r, int w) {
-            return G::interior_row(r) + G::col(w + G::PL);
-        }
-    };
-    const int tid = threadIdx.x;
+    constexpr int ITERS = (PB * G::IPP + NT - 1) / NT;
+    const unsigned tid = threadIdx.x;
+    const unsigned pstride = (unsigned)C * (H * W);  // elements between images of one channel
 
     // weights of this channel, duplicates folded into their representative tap
     float wv[K];
@@ -192,80 +272,110 @@ __device__ __forceinline__ void run_canonical(const T *__restrict__ src, const f
         constexpr int r = G::plan.rep[s];
         if constexpr (r >= 0 && r != s) wv[r] += wv[s];
     });
+    // folded sums are uniform: move them back to scalar registers
+    static_for<K>([&](auto s) {
+        if constexpr (s > 0 && G::plan.rep[s] >= 0 && G::plan.rep[s] != s) {
+            constexpr int r = G::plan.rep[s];
+            wv[r] = __builtin_bit_cast(
+                float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, wv[r])));
+        }
+    });
     const float bv = (OP == OP_FPROP && bias != nullptr) ? bias[c] : 0.f;
 
     // zero the staging area once; interiors are overwritten per batch, halos stay zero
-    for (int i = tid; i < PB * PLS; i += NT) lds[i] = 0.f;
+    for (unsigned i = tid; i < PB * PLS; i += NT) lds[i] = 0.f;
 
-    Stager<T, H, W, PB, NT, PLS, Map> st;
-    st.prefetch(src, c, C, n0, n1);
-    for (int nb = n0; nb < n1; nb += PB) {
+    const T *sbase = src + (size_t)c * (H * W);
+    T *dbase = dst + (size_t)c * (H * W);
+
+    // Two register sets keep two batches in flight from HBM while a third is being computed.
+    auto process = [&](auto &stg, int nb) {
+        const int nvalid = n1 - nb;
+        set_progress_priority(nvalid, n1 - n0);
         __syncthreads();  // previous batch fully consumed (first pass: zero fill done)
-        st.commit(lds, nb, n1);
+        stg.template commit<GeoMap<G>, PLS>(lds, nvalid);
         __syncthreads();
-        if (nb + PB < n1) st.prefetch(src, c, C, nb + PB, n1);
-
-        for (int item = tid; item < PB * G::IPP; item += NT) {
-            const int pl = item / G::IPP, it = item % G::IPP;
-            const int rb = it / G::IPR, j = it % G::IPR;
-            if (nb + pl >= n1) break;
-            const float *base = lds + pl * PLS + rb * (G::LR * G::RS) + j;
-            float acc[L];
+        if (nb + 2 * PB < n1)
+            stg.prefetch(sbase + (size_t)(nb + 2 * PB) * pstride, pstride, n1 - nb - 2 * PB);
+        T *obase = dbase + (size_t)nb * pstride;  // uniform
 #pragma unroll
-            for (int l = 0; l < L; l++) acc[l] = bv;
-            static_for<G::plan.nsrc>([&](auto m) {
-                constexpr int off = G::imm(G::plan.sh[m], G::plan.sw[m]);
-                const float v = base[off];
-                static_for<L>([&](auto l) {
-                    constexpr int t = G::plan.user[m][l];
-                    if constexpr (t >= 0) acc[l] = __builtin_fmaf(v, wv[t], acc[l]);
+        for (int iter = 0; iter < ITERS; iter++) {
+            const unsigned item = tid + iter * NT;
+            const unsigned pl = item / G::IPP, it = item % G::IPP;
+            const unsigned rb = it / G::IPR, j = it % G::IPR;
+            if (item < PB * G::IPP && (int)pl < nvalid) {
+                const float *base = lds + (pl * PLS + rb * (G::LR * G::RS) + j);
+                float acc[L];
+#pragma unroll
+                for (int l = 0; l < L; l++) acc[l] = bv;
+                static_for<G::plan.nsrc>([&](auto m) {
+                    constexpr int off = G::imm(G::plan.sh[m], G::plan.sw[m]);
+                    const float v = base[off];
+                    static_for<L>([&](auto l) {
+                        constexpr int t = G::plan.user[m][l];
+                        if constexpr (t >= 0) acc[l] = __builtin_fmaf(v, wv[t], acc[l]);
+                    });
                 });
-            });
-            T *out = dst + ((size_t)(nb + pl) * C + c) * (H * W);
-            if constexpr (G::CLS == CLS_H) {
-                T *o = out + rb * W + j * L;
-                if constexpr (L == 4) {
-                    Vec4<T> r;
-                    r.set(acc[0], acc[1], acc[2], acc[3]);
-                    r.store(o);
+                if constexpr (G::CLS == CLS_H) {
+                    T *o = obase + (pl * pstride + rb * W + j * L);
+                    if constexpr (L == 4) {
+                        Vec4<T> r;
+                        r.set(acc[0], acc[1], acc[2], acc[3]);
+                        r.store(o);
+                    } else {
+#pragma unroll
+                        for (int l = 0; l < L; l++) st_out(o + l, from_float<T>(acc[l]));
+                    }
+                } else if constexpr (G::CLS == CLS_V) {
+                    T *o = obase + (pl * pstride + rb * (L * W) + j);
+#pragma unroll
+                    for (int l = 0; l < L; l++)
+                        if (H % L == 0 || rb * L + l < H) st_out(o + l * W, from_float<T>(acc[l]));
                 } else {
+                    // output l sits at row rb*L + P0 + l*EH, column j - Q0 + l
+                    T *o = obase + (pl * pstride + rb * (L * W) + j);
 #pragma unroll
-                    for (int l = 0; l < L; l++) o[l] = from_float<T>(acc[l]);
-                }
-            } else if constexpr (G::CLS == CLS_V) {
-#pragma unroll
-                for (int l = 0; l < L; l++)
-                    if (H % L == 0 || rb * L + l < H) out[(rb * L + l) * W + j] = from_float<T>(acc[l]);
-            } else {
-                const int p0 = rb * L + G::P0, q0 = j - G::Q0;
-#pragma unroll
-                for (int l = 0; l < L; l++) {
-                    const int p = p0 + l * G::EH, q = q0 + l;
-                    if (q >= 0 && q < W && (H % L == 0 || p < H)) out[p * W + q] = from_float<T>(acc[l]);
+                    for (int l = 0; l < L; l++) {
+                        const unsigned q = j + (unsigned)(l - G::Q0);  // wraps when negative
+                        if (q < W && (H % L == 0 || rb * L + G::P0 + l * G::EH < H))
+                            st_out(o + ((G::P0 + l * G::EH) * W + l - G::Q0), from_float<T>(acc[l]));
+                    }
                 }
             }
         }
+    };
+    for (int nb = n0; nb < n1; nb += 2 * PB) {
+        process(sg.a, nb);
+        if (nb + PB < n1) process(sg.b, nb + PB);
     }
 }
 
 // ---------------------------------------------------------------------------------------------
 // table-driven body (any angle): same staging with a square halo, taps from the device table
 // ---------------------------------------------------------------------------------------------
+template <int K, int H, int W>
+struct TableMap {
+    static constexpr int PAD = table_pad<K, H, W>();
+    static constexpr int PL = (PAD + 3) & ~3;
+    static constexpr int RS = W + PL + PAD;
+    static __device__ __forceinline__ unsigned index(unsigned r, unsigned w) {
+        return (r + PAD) * RS + w + PL;
+    }
+    static constexpr int step(int e) { return e; }
+};
+
 template <int OP, typename T, int K, int H, int W>
 __device__ __forceinline__ void run_table(const T *__restrict__ src, const float *__restrict__ wt,
                                           const float *__restrict__ bias,
                                           const int8_t *__restrict__ dhdw, T *__restrict__ dst,
-                                          float *lds, int c, int C, int n0, int n1) {
+                                          float *lds, int c, int C, int n0, int n1,
+                                          ConvStagers<T, H, W> &sg) {
     constexpr int PB = Tile<H, W>::PB, NT = Tile<H, W>::NT;
-    constexpr int PAD = table_pad<K, H, W>();
-    constexpr int PL = (PAD + 3) & ~3;
-    constexpr int RS = W + PL + PAD;
+    using Map = TableMap<K, H, W>;
     constexpr int PLS = plane_floats<K, H, W>();
-    static_assert((H + 2 * PAD) * RS <= PLS, "table body staging must fit the plane stride");
-    struct Map {
-        static __device__ __forceinline__ int index(int r, int w) { return (r + PAD) * RS + w + PL; }
-    };
-    const int tid = threadIdx.x;
+    static_assert((H + 2 * Map::PAD) * Map::RS <= PLS, "table body staging must fit the plane stride");
+    const unsigned tid = threadIdx.x;
+    const unsigned pstride = (unsigned)C * (H * W);
     // live taps of this channel as LDS offsets, with their weights (dead taps never reach the
     // plane and are skipped); kept in LDS behind the planes
     int *toff = reinterpret_cast<int *>(lds + PB * PLS);
@@ -276,51 +386,230 @@ __device__ __forceinline__ void run_table(const T *__restrict__ src, const float
         for (int s = 0; s < K; s++) {
             const int dh = dhdw[((size_t)c * K + s) * 2], dw = dhdw[((size_t)c * K + s) * 2 + 1];
             if (dh >= H || dh <= -H || dw >= W || dw <= -W) continue;
-            toff[nl] = (OP == OP_DGRAD ? -1 : 1) * (dh * RS + dw);
+            toff[nl] = (OP == OP_DGRAD ? -1 : 1) * (dh * Map::RS + dw);
             twt[nl] = wt[(size_t)c * K + s];
             nl++;
         }
         nlive_s = nl;
     }
     const float bv = (OP == OP_FPROP && bias != nullptr) ? bias[c] : 0.f;
-    for (int i = tid; i < PB * PLS; i += NT) lds[i] = 0.f;
-    Stager<T, H, W, PB, NT, PLS, Map> st;
-    st.prefetch(src, c, C, n0, n1);
-    for (int nb = n0; nb < n1; nb += PB) {
+    for (unsigned i = tid; i < PB * PLS; i += NT) lds[i] = 0.f;
+    const T *sbase = src + (size_t)c * (H * W);
+    T *dbase = dst + (size_t)c * (H * W);
+    auto process = [&](auto &stg, int nb) {
+        const int nvalid = n1 - nb;
         __syncthreads();
-        st.commit(lds, nb, n1);
+        stg.template commit<Map, PLS>(lds, nvalid);
         __syncthreads();
-        if (nb + PB < n1) st.prefetch(src, c, C, nb + PB, n1);
+        if (nb + 2 * PB < n1)
+            stg.prefetch(sbase + (size_t)(nb + 2 * PB) * pstride, pstride, nvalid - 2 * PB);
         const int nlive = nlive_s;
-        for (int f = tid; f < PB * H * W; f += NT) {
-            const int pl = f / (H * W), g = f % (H * W);
-            if (nb + pl >= n1) break;
+        T *obase = dbase + (size_t)nb * pstride;
+        for (unsigned f = tid; f < PB * H * W; f += NT) {
+            const unsigned pl = f / (H * W), g = f % (H * W);
+            if ((int)pl >= nvalid) break;
             const float *base = lds + pl * PLS + Map::index(g / W, g % W);
             float acc = bv;
             for (int s = 0; s < nlive; s++) acc = __builtin_fmaf(base[toff[s]], twt[s], acc);
-            dst[((size_t)(nb + pl) * C + c) * (H * W) + g] = from_float<T>(acc);
+            st_out(obase + (pl * pstride + g), from_float<T>(acc));
         }
+    };
+    for (int nb = n0; nb < n1; nb += 2 * PB) {
+        process(sg.a, nb);
+        if (nb + PB < n1) process(sg.b, nb + PB);
     }
 }
 
-// LDS bytes a launch of plane_kernel<.., K, H, W> needs
-template <int K, int H, int W>
-constexpr size_t plane_kernel_lds_bytes() {
-    return ((size_t)Tile<H, W>::PB * plane_floats<K, H, W>() + 2 * K) * sizeof(float);
+// ---------------------------------------------------------------------------------------------
+// wgrad: dw[c,s] = sum over n,p,q of x[n,c,p+dh(s),q+dw(s)] * dy[n,c,p,q]
+// ---------------------------------------------------------------------------------------------
+// Wave64 sum with DPP row shifts and row broadcasts (no LDS traffic); the total lands in lane 63.
+__device__ __forceinline__ float wave_sum_dpp(float v) {
+#define DWO_DPP_ADD(ctrl, row_mask)                                                              \
+    v += __builtin_bit_cast(                                                                     \
+        float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), ctrl, row_mask, 0xf, true))
+    DWO_DPP_ADD(0x111, 0xf);  // row_shr:1
+    DWO_DPP_ADD(0x112, 0xf);  // row_shr:2
+    DWO_DPP_ADD(0x114, 0xf);  // row_shr:4
+    DWO_DPP_ADD(0x118, 0xf);  // row_shr:8  -> lane 15 of each row holds the row total
+    DWO_DPP_ADD(0x142, 0xa);  // row_bcast:15 into rows 1 and 3
+    DWO_DPP_ADD(0x143, 0xc);  // row_bcast:31 into rows 2 and 3
+#undef DWO_DPP_ADD
+    return v;
 }
 
-template <int OP, typename T, int K, int H, int W>
-__global__ __launch_bounds__((Tile<H, W>::NT)) void plane_kernel(
-    const T *__restrict__ src, const float *__restrict__ wt, const float *__restrict__ bias,
-    const void *__restrict__ blob, T *__restrict__ dst, int N, int C, int G) {
+// Workgroup epilogue: per-thread accumulators acc[0..NV) -> wave totals (DPP) -> LDS -> one
+// partial per value written to part[(c*(K+1) + s) * NG + group].  `slot_of(s)` maps tap s to the
+// accumulator that holds its sum (-1: the tap never reaches the plane, its gradient is zero).
+template <int K, int NT, class SlotOf>
+__device__ __forceinline__ void wgrad_epilogue(float (&acc)[K + 1], float *lds, float *__restrict__ part,
+                                               int c, int group, int NG, SlotOf slot_of) {
+    constexpr int NW = NT / 64;
+    __syncthreads();  // staged planes are dead from here on
+#pragma unroll
+    for (int s = 0; s <= K; s++) {
+        const float t = wave_sum_dpp(acc[s]);
+        if ((threadIdx.x & 63) == 63) lds[(threadIdx.x >> 6) * (K + 1) + s] = t;
+    }
+    __syncthreads();
+    if (threadIdx.x <= K) {
+        const int slot = threadIdx.x == K ? K : slot_of(threadIdx.x);
+        float t = 0.f;
+        if (slot >= 0)
+            for (int w = 0; w < NW; w++) t += lds[w * (K + 1) + slot];
+        part[((size_t)c * (K + 1) + threadIdx.x) * NG + group] = t;
+    }
+}
+
+// dy planes are staged unpadded right behind the x planes and the tap tables
+template <int H, int W>
+struct FlatMap {
+    static __device__ __forceinline__ unsigned index(unsigned r, unsigned w) { return r * W + w; }
+    static constexpr int step(int e) { return e; }
+};
+template <int K, int H, int W>
+constexpr int wgrad_dy_offset() {
+    return (Tile<H, W>::PB * plane_floats<K, H, W>() + 2 * K + 3) & ~3;
+}
+
+template <int O, typename T, int K, int H, int W>
+__device__ __forceinline__ void run_canonical_wgrad(const T *__restrict__ x, const T *__restrict__ dy,
+                                                    float *__restrict__ part, float *lds, int c,
+                                                    int C, int n0, int n1, int group, int NG) {
+    constexpr int L = tile_L<H, W>(O);
+    constexpr int PB = Tile<H, W>::PB, NT = Tile<H, W>::NT;
+    using G = Geo<O, K, L, H, W>;
+    constexpr int PLS = plane_floats<K, H, W>();
+    constexpr int ITERS = (PB * G::IPP + NT - 1) / NT;
+    const unsigned tid = threadIdx.x;
+    const unsigned pstride = (unsigned)C * (H * W);
+    for (unsigned i = tid; i < PB * PLS; i += NT) lds[i] = 0.f;
+    const T *xbase = x + (size_t)c * (H * W);
+    const T *gbase = dy + (size_t)c * (H * W);
+    float *ldy = lds + wgrad_dy_offset<K, H, W>();
+
+    float acc[K + 1];  // acc[s] for representative taps s, acc[K] = sum of dy (bias gradient)
+#pragma unroll
+    for (int s = 0; s <= K; s++) acc[s] = 0.f;
+
+    Stager<T, H, W, PB, NT> sx, sg;
+    sx.prefetch(xbase + (size_t)n0 * pstride, pstride, n1 - n0);
+    sg.prefetch(gbase + (size_t)n0 * pstride, pstride, n1 - n0);
+    for (int nb = n0; nb < n1; nb += PB) {
+        const int nvalid = n1 - nb;
+        __syncthreads();
+        sx.template commit<GeoMap<G>, PLS>(lds, nvalid);
+        sg.template commit<FlatMap<H, W>, H * W>(ldy, nvalid);
+        __syncthreads();
+        if (nb + PB < n1) {
+            sx.prefetch(xbase + (size_t)(nb + PB) * pstride, pstride, nvalid - PB);
+            sg.prefetch(gbase + (size_t)(nb + PB) * pstride, pstride, nvalid - PB);
+        }
+#pragma unroll
+        for (int it = 0; it < ITERS; it++) {
+            const unsigned item = tid + it * NT;
+            const unsigned pl = item / G::IPP, ii = item % G::IPP;
+            const unsigned rb = ii / G::IPR, j = ii % G::IPR;
+            if (item < PB * G::IPP && (int)pl < nvalid) {
+                // dy of the item's L outputs (zero where the output does not exist)
+                float d[L];
+                const float *g = ldy + pl * (H * W);
+                if constexpr (G::CLS == CLS_H) {
+#pragma unroll
+                    for (int l = 0; l < L; l++) d[l] = g[rb * W + j * L + l];
+                } else if constexpr (G::CLS == CLS_V) {
+#pragma unroll
+                    for (int l = 0; l < L; l++)
+                        d[l] = (H % L == 0 || rb * L + l < H) ? g[(rb * L + l) * W + j] : 0.f;
+                } else {
+#pragma unroll
+                    for (int l = 0; l < L; l++) {
+                        const unsigned q = j + (unsigned)(l - G::Q0);
+                        const bool ok = q < W && (H % L == 0 || rb * L + G::P0 + l * G::EH < H);
+                        d[l] = ok ? g[(int)(rb * (L * W) + j) + (G::P0 + l * G::EH) * W + l - G::Q0] : 0.f;
+                    }
+                }
+                const float *base = lds + (pl * PLS + rb * (G::LR * G::RS) + j);
+                static_for<G::plan.nsrc>([&](auto m) {
+                    constexpr int off = G::imm(G::plan.sh[m], G::plan.sw[m]);
+                    const float v = base[off];
+                    static_for<L>([&](auto l) {
+                        constexpr int t = G::plan.user[m][l];
+                        if constexpr (t >= 0) acc[t] = __builtin_fmaf(v, d[l], acc[t]);
+                    });
+                });
+#pragma unroll
+                for (int l = 0; l < L; l++) acc[K] += d[l];
+            }
+        }
+    }
+    wgrad_epilogue<K, NT>(acc, lds, part, c, group, NG,
+                          [](int s) { return (int)G::plan.rep[s]; });
+}
+
+// table-driven wgrad body (any angle)
+template <typename T, int K, int H, int W>
+__device__ __forceinline__ void run_table_wgrad(const T *__restrict__ x, const T *__restrict__ dy,
+                                                const int8_t *__restrict__ dhdw,
+                                                float *__restrict__ part, float *lds, int c, int C,
+                                                int n0, int n1, int group, int NG) {
+    constexpr int PB = Tile<H, W>::PB, NT = Tile<H, W>::NT;
+    using Map = TableMap<K, H, W>;
+    constexpr int PLS = plane_floats<K, H, W>();
+    const unsigned tid = threadIdx.x;
+    const unsigned pstride = (unsigned)C * (H * W);
+    int *toff = reinterpret_cast<int *>(lds + PB * PLS);  // LDS offset per tap; dead taps read the
+    int *tlive = toff + K;                                 // centre and are zeroed at the end
+    if (tid < K) {
+        const int dh = dhdw[((size_t)c * K + tid) * 2], dw = dhdw[((size_t)c * K + tid) * 2 + 1];
+        const bool dead = dh >= H || dh <= -H || dw >= W || dw <= -W;
+        toff[tid] = dead ? 0 : dh * Map::RS + dw;
+        tlive[tid] = dead ? -1 : (int)tid;
+    }
+    for (unsigned i = tid; i < PB * PLS; i += NT) lds[i] = 0.f;
+    float acc[K + 1];
+#pragma unroll
+    for (int s = 0; s <= K; s++) acc[s] = 0.f;
+    const T *xbase = x + (size_t)c * (H * W);
+    const T *gbase = dy + (size_t)c * (H * W);
+    Stager<T, H, W, PB, NT> st;
+    st.prefetch(xbase + (size_t)n0 * pstride, pstride, n1 - n0);
+    for (int nb = n0; nb < n1; nb += PB) {
+        const int nvalid = n1 - nb;
+        __syncthreads();
+        st.template commit<Map, PLS>(lds, nvalid);
+        __syncthreads();
+        if (nb + PB < n1) st.prefetch(xbase + (size_t)(nb + PB) * pstride, pstride, nvalid - PB);
+        const T *gb = gbase + (size_t)nb * pstride;
+        for (unsigned f = tid; f < PB * H * W; f += NT) {
+            const unsigned pl = f / (H * W), g = f % (H * W);
+            if ((int)pl >= nvalid) break;
+            const float gy = to_float(gb[pl * pstride + g]);
+            const float *base = lds + pl * PLS + Map::index(g / W, g % W);
+#pragma unroll
+            // (offsets are re-read from LDS per tap: keeping all K of them in registers next to
+            // the K accumulators would cost occupancy for every channel, canonical ones included)
+            for (int s = 0; s < K; s++)
+                acc[s] = __builtin_fmaf(base[*(volatile int *)&toff[s]], gy, acc[s]);
+            acc[K] += gy;
+        }
+    }
+    wgrad_epilogue<K, NT>(acc, lds, part, c, group, NG, [&](int s) { return tlive[s]; });
+}
+
+template <typename T, int K, int H, int W>
+__global__ __launch_bounds__((Tile<H, W>::NT)) __attribute__((amdgpu_waves_per_eu(DWO_WPE_WGRAD, 8))) void plane_wgrad_kernel(
+    const T *__restrict__ x, const T *__restrict__ dy, const void *__restrict__ blob,
+    float *__restrict__ part, int N, int C, int NG) {
     extern __shared__ float lds[];
-    const int c = blockIdx.x % C;
-    const int n0 = (blockIdx.x / C) * G;
-    const int n1 = min(n0 + G, N);
+    int c, group;
+    plane_task(C, NG, c, group);
+    int n0, n1;
+    group_range<Tile<H, W>::PB>(N, NG, group, n0, n1);
     const int cls = taps_class(blob, C, K)[c];
-#define DWO_CASE(O)                                                                  \
-    case O:                                                                          \
-        run_canonical<O, OP, T, K, H, W>(src, wt, bias, dst, lds, c, C, n0, n1);      \
+#define DWO_CASE(O)                                                                      \
+    case O:                                                                              \
+        run_canonical_wgrad<O, T, K, H, W>(x, dy, part, lds, c, C, n0, n1, group, NG);    \
         break;
     switch (cls) {
         DWO_CASE(0)
@@ -332,9 +621,123 @@ __global__ __launch_bounds__((Tile<H, W>::NT)) void plane_kernel(
         DWO_CASE(6)
         DWO_CASE(7)
         default:
-            run_table<OP, T, K, H, W>(src, wt, bias, taps_dhdw(blob), dst, lds, c, C, n0, n1);
+            run_table_wgrad<T, K, H, W>(x, dy, taps_dhdw(blob), part, lds, c, C, n0, n1, group, NG);
     }
 #undef DWO_CASE
+}
+
+// LDS bytes a launch of plane_kernel / plane_wgrad_kernel<.., K, H, W> needs
+template <int K, int H, int W>
+constexpr size_t plane_kernel_lds_bytes() {
+    return ((size_t)Tile<H, W>::PB * plane_floats<K, H, W>() + 2 * K) * sizeof(float);
+}
+template <int K, int H, int W>
+constexpr size_t plane_wgrad_lds_bytes() {
+    return ((size_t)wgrad_dy_offset<K, H, W>() + Tile<H, W>::PB * H * W) * sizeof(float);
+}
+
+#ifdef DWO_DBG_TIMING
+__device__ long long g_dbg[8192 * 4];
+#endif
+
+template <int OP, typename T, int K, int H, int W>
+__global__ __launch_bounds__((Tile<H, W>::NT)) __attribute__((amdgpu_waves_per_eu(DWO_WPE, 8))) void plane_kernel(
+    const T *__restrict__ src, const float *__restrict__ wt, const float *__restrict__ bias,
+    const void *__restrict__ blob, T *__restrict__ dst, int N, int C, int groups) {
+    extern __shared__ float lds[];
+    int c, group;
+    plane_task(C, groups, c, group);
+    int n0, n1;
+    group_range<Tile<H, W>::PB>(N, groups, group, n0, n1);
+#ifdef DWO_DBG_TIMING
+    const long long t_start = wall_clock64();
+#endif
+    ConvStagers<T, H, W> sg;
+    sg.start(src, c, C, n0, n1);  // HBM latency overlaps the class lookup, weights and zero fill
+    const int cls = taps_class(blob, C, K)[c];
+#define DWO_CASE(O)                                                                  \
+    case O:                                                                          \
+        run_canonical<O, OP, T, K, H, W>(src, wt, bias, dst, lds, c, C, n0, n1, sg);  \
+        break;
+    switch (cls) {
+        DWO_CASE(0)
+        DWO_CASE(1)
+        DWO_CASE(2)
+        DWO_CASE(3)
+        DWO_CASE(4)
+        DWO_CASE(5)
+        DWO_CASE(6)
+        DWO_CASE(7)
+        default:
+            run_table<OP, T, K, H, W>(src, wt, bias, taps_dhdw(blob), dst, lds, c, C, n0, n1, sg);
+    }
+#undef DWO_CASE
+#ifdef DWO_DBG_TIMING
+    if ((threadIdx.x & 63) == 0 && blockIdx.x < 1024) {
+        unsigned hwid;
+        asm volatile("s_getreg_b32 %0, hwreg(HW_REG_HW_ID)" : "=s"(hwid));
+        g_dbg[8192 * 2 + blockIdx.x * 8 + (threadIdx.x >> 6)] = hwid;
+    }
+    if (threadIdx.x == 0 && blockIdx.x < 4096) {
+        unsigned hwid;
+        asm volatile("s_getreg_b32 %0, hwreg(HW_REG_HW_ID)" : "=s"(hwid));
+        unsigned xcc;
+        asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
+        g_dbg[blockIdx.x * 4 + 0] = t_start;
+        g_dbg[blockIdx.x * 4 + 1] = wall_clock64();
+        g_dbg[blockIdx.x * 4 + 2] = ((long long)xcc << 32) | hwid;
+        g_dbg[blockIdx.x * 4 + 3] = ((long long)cls << 32) | (unsigned)(n1 - n0);
+    }
+#endif
+}
+
+// ---------------------------------------------------------------------------------------------
+// host launchers (instantiated per element type and plane extent in dwo_inst.hip)
+// ---------------------------------------------------------------------------------------------
+// Workgroups that can be resident at once on the current device for a kernel.
+template <class Kern>
+int resident_slots(Kern kern, int block, size_t lds) {
+    int dev = 0, cus = 0, per_cu = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
+        hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kern, block, lds) != hipSuccess ||
+        cus < 1 || per_cu < 1)
+        return 1024;
+    return cus * per_cu;
+}
+
+template <typename T, int K, int H, int W>
+int launch_plane_conv(int op, const void *src, const float *w, const float *bias, const void *taps,
+                      void *dst, int N, int C, hipStream_t st) {
+    constexpr int NT = Tile<H, W>::NT;
+    const size_t lds = plane_kernel_lds_bytes<K, H, W>();
+    static const int slots_f = resident_slots(plane_kernel<OP_FPROP, T, K, H, W>, NT, lds);
+    static const int dbg_groups = getenv("DWO_GROUPS") ? atoi(getenv("DWO_GROUPS")) : 0;
+    const int groups = dbg_groups ? dbg_groups : plane_groups(N, C, Tile<H, W>::PB, slots_f);
+    const dim3 grid(C * groups), block(NT);
+    if (op == OP_FPROP)
+        plane_kernel<OP_FPROP, T, K, H, W><<<grid, block, lds, st>>>((const T *)src, w, bias, taps,
+                                                                   (T *)dst, N, C, groups);
+    else
+        plane_kernel<OP_DGRAD, T, K, H, W><<<grid, block, lds, st>>>((const T *)src, w, bias, taps,
+                                                                   (T *)dst, N, C, groups);
+    const hipError_t e = hipGetLastError();
+    return e == hipSuccess ? 0 : (int)e;
+}
+
+// Writes NG = *groups_out partials per (channel, tap) into part[(c*(K+1)+s)*NG + g].
+template <typename T, int K, int H, int W>
+int launch_plane_wgrad(const void *x, const void *dy, const void *taps, float *part, int N, int C,
+                       int *groups_out, hipStream_t st) {
+    constexpr int NT = Tile<H, W>::NT;
+    const size_t lds = plane_wgrad_lds_bytes<K, H, W>();
+    static const int slots = resident_slots(plane_wgrad_kernel<T, K, H, W>, NT, lds);
+    const int groups = plane_groups(N, C, Tile<H, W>::PB, slots);
+    *groups_out = groups;
+    plane_wgrad_kernel<T, K, H, W><<<dim3(C * groups), dim3(NT), lds, st>>>(
+        (const T *)x, (const T *)dy, taps, part, N, C, groups);
+    const hipError_t e = hipGetLastError();
+    return e == hipSuccess ? 0 : (int)e;
 }
 
 }  // namespace dwo

@@ -87,6 +87,18 @@ def test_stage_shapes_k31(oracle, C, HW, nhwc, dtype):
     _case(oracle, 4, C, HW, HW, 31, 1, dtype, nhwc, canonical_theta(C), seed=C + HW)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("C,HW", [(40, 56), (40, 28), (72, 14), (100, 7)])
+def test_stage_shapes_mixed_angles(oracle, C, HW, dtype):
+    """Stage plane extents with arbitrary angles mixed among canonical ones (a workgroup picks
+    the compile-time or the table-driven body per channel), odd batch and channel counts."""
+    rng = np.random.default_rng(HW)
+    theta = canonical_theta(C)
+    theta[1::3] = rng.uniform(-math.pi, 2 * math.pi, len(theta[1::3])).astype(np.float32)
+    _case(oracle, 5, C, HW, HW, 31, 1, dtype, False, theta, seed=HW * 3)
+    _case(oracle, 3, C, HW, HW, 31, 1, dtype, False, grouped_theta(C, 0.5), seed=HW * 5)
+
+
 @pytest.mark.parametrize("nhwc", [False, True], ids=["nchw", "nhwc"])
 @pytest.mark.parametrize("K", [7, 13, 15, 27, 31])
 def test_kernel_sizes_grouped_theta(oracle, K, nhwc):
