@@ -49,6 +49,8 @@ def main():
     ap.add_argument("--theta", default="roundrobin", choices=["roundrobin", "grouped"])
     ap.add_argument("--kernel-iters", type=int, default=30,
                     help="back-to-back launches per (shape, op) for the per-kernel timings")
+    ap.add_argument("--kernel-repeats", type=int, default=7,
+                    help="repeats of the per-kernel measurement (the median is reported)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--only", default="", help="restrict the per-kernel table, e.g. 96x56:fprop")
     args = ap.parse_args()
@@ -168,13 +170,16 @@ def main():
             for i in range(3):
                 run_op(name, si, i)
             torch.cuda.synchronize()
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            e0.record(stream)
-            for i in range(args.kernel_iters):
-                run_op(name, si, i)
-            e1.record(stream)
-            torch.cuda.synchronize()
-            us = e0.elapsed_time(e1) * 1e3 / args.kernel_iters
+            reps = []
+            for _ in range(args.kernel_repeats):
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record(stream)
+                for i in range(args.kernel_iters):
+                    run_op(name, si, i)
+                e1.record(stream)
+                torch.cuda.synchronize()
+                reps.append(e0.elapsed_time(e1) * 1e3 / args.kernel_iters)
+            us = sorted(reps)[len(reps) // 2]  # median of the repeats
             ab = algorithmic_bytes(name, BATCH, C, HW, HW, KSIZE, b)
             gbs = ab / (us * 1e-6) / 1e9
             detail[key] = {"us": round(us, 2), "GB/s": round(gbs, 1),

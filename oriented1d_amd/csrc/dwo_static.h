@@ -195,24 +195,6 @@ struct GeoMap {
     }
 };
 
-// Wave priority from the fraction of the workgroup's images still to do.  The hardware issues
-// oldest-wave-first, so of the workgroups sharing a CU the youngest would otherwise starve, end
-// last and run its tail alone at low occupancy; raising the priority of whoever has most work
-// left keeps co-resident workgroups in step so that they finish together.
-__device__ __forceinline__ void set_progress_priority(int remaining, int total) {
-#ifndef DWO_NO_PRIO
-    const int level = (remaining * 4 - 1) / total;  // 3 .. 0
-    if (level >= 3)
-        __builtin_amdgcn_s_setprio(3);
-    else if (level == 2)
-        __builtin_amdgcn_s_setprio(2);
-    else if (level == 1)
-        __builtin_amdgcn_s_setprio(1);
-    else
-        __builtin_amdgcn_s_setprio(0);
-#endif
-}
-
 // Workgroup -> (channel, image group).  Hardware hands consecutive workgroup ids to the eight
 // XCDs round-robin and fills the CUs of an XCD in order, while orientation (hence cost) often
 // repeats with period 8 over the channels; rotating the task id inside every aligned block of
@@ -231,6 +213,32 @@ __device__ __forceinline__ void group_range(int N, int groups, int g, int &n0, i
     const int nbatch = (N + PB - 1) / PB;
     n0 = (int)(((long)g * nbatch) / groups) * PB;
     n1 = min((int)(((long)(g + 1) * nbatch) / groups) * PB, N);
+}
+
+// V and D class items produce one element per lane and row.  As 2-byte stores these run far
+// below the rate of wider ones, so for 16-bit activations their results go through an unpadded fp32 out-tile in LDS (behind the
+// planes and the tap tables) and leave as 16/8-byte non-temporal stores one batch later.
+template <int K, int H, int W>
+constexpr int out_tile_offset() {
+    return (Tile<H, W>::PB * plane_floats<K, H, W>() + 2 * K + 3) & ~3;
+}
+template <typename T, int H, int W>
+constexpr bool use_out_tile() {
+    return sizeof(T) < 4 && (H * W) % 4 == 0;  // 4-byte stores run at full rate as they are
+}
+template <typename T, int H, int W, int PB, int NT>
+__device__ __forceinline__ void flush_out_tile(const float *lout, T *__restrict__ obase,
+                                               unsigned pstride, int nvalid) {
+    constexpr int FP = H * W / 4;
+    for (unsigned f = threadIdx.x; f < PB * FP; f += NT) {
+        const unsigned pl = f / FP, g = f % FP;
+        if ((int)pl < nvalid) {
+            const float4 v = *reinterpret_cast<const float4 *>(lout + f * 4);
+            Vec4<T> r;
+            r.set(v.x, v.y, v.z, v.w);
+            r.store(obase + (pl * pstride + g * 4));
+        }
+    }
 }
 
 // The two register sets of the fprop/dgrad pipeline; start() issues the loads of the first two
@@ -288,11 +296,17 @@ __device__ __forceinline__ void run_canonical(const T *__restrict__ src, const f
     const T *sbase = src + (size_t)c * (H * W);
     T *dbase = dst + (size_t)c * (H * W);
 
+    constexpr bool TILE = G::CLS != CLS_H && use_out_tile<T, H, W>();
+    float *lout = lds + out_tile_offset<K, H, W>();
+
     // Two register sets keep two batches in flight from HBM while a third is being computed.
     auto process = [&](auto &stg, int nb) {
         const int nvalid = n1 - nb;
-        set_progress_priority(nvalid, n1 - n0);
         __syncthreads();  // previous batch fully consumed (first pass: zero fill done)
+        if constexpr (TILE) {
+            if (nb > n0)
+                flush_out_tile<T, H, W, PB, NT>(lout, dbase + (size_t)(nb - PB) * pstride, pstride, PB);
+        }
         stg.template commit<GeoMap<G>, PLS>(lds, nvalid);
         __syncthreads();
         if (nb + 2 * PB < n1)
@@ -327,26 +341,43 @@ __device__ __forceinline__ void run_canonical(const T *__restrict__ src, const f
                         for (int l = 0; l < L; l++) st_out(o + l, from_float<T>(acc[l]));
                     }
                 } else if constexpr (G::CLS == CLS_V) {
-                    T *o = obase + (pl * pstride + rb * (L * W) + j);
+                    // output l sits at row rb*L + l, column j
 #pragma unroll
                     for (int l = 0; l < L; l++)
-                        if (H % L == 0 || rb * L + l < H) st_out(o + l * W, from_float<T>(acc[l]));
+                        if (H % L == 0 || rb * L + l < H) {
+                            if constexpr (TILE)
+                                lout[pl * (H * W) + rb * (L * W) + j + l * W] = acc[l];
+                            else
+                                st_out(obase + (pl * pstride + rb * (L * W) + j) + l * W,
+                                       from_float<T>(acc[l]));
+                        }
                 } else {
                     // output l sits at row rb*L + P0 + l*EH, column j - Q0 + l
-                    T *o = obase + (pl * pstride + rb * (L * W) + j);
 #pragma unroll
                     for (int l = 0; l < L; l++) {
                         const unsigned q = j + (unsigned)(l - G::Q0);  // wraps when negative
-                        if (q < W && (H % L == 0 || rb * L + G::P0 + l * G::EH < H))
-                            st_out(o + ((G::P0 + l * G::EH) * W + l - G::Q0), from_float<T>(acc[l]));
+                        const int doff = (G::P0 + l * G::EH) * W + l - G::Q0;
+                        if (q < W && (H % L == 0 || rb * L + G::P0 + l * G::EH < H)) {
+                            if constexpr (TILE)
+                                lout[(int)(pl * (H * W) + rb * (L * W) + j) + doff] = acc[l];
+                            else
+                                st_out(obase + (pl * pstride + rb * (L * W) + j) + doff,
+                                       from_float<T>(acc[l]));
+                        }
                     }
                 }
             }
         }
     };
-    for (int nb = n0; nb < n1; nb += 2 * PB) {
+    int nb = n0;
+    for (; nb < n1; nb += 2 * PB) {
         process(sg.a, nb);
         if (nb + PB < n1) process(sg.b, nb + PB);
+    }
+    if constexpr (TILE) {
+        const int last = n0 + ((n1 - n0 - 1) / PB) * PB;  // first image of the final batch
+        __syncthreads();
+        flush_out_tile<T, H, W, PB, NT>(lout, dbase + (size_t)last * pstride, pstride, n1 - last);
     }
 }
 
@@ -627,9 +658,10 @@ __global__ __launch_bounds__((Tile<H, W>::NT)) __attribute__((amdgpu_waves_per_e
 }
 
 // LDS bytes a launch of plane_kernel / plane_wgrad_kernel<.., K, H, W> needs
-template <int K, int H, int W>
+template <typename T, int K, int H, int W>
 constexpr size_t plane_kernel_lds_bytes() {
-    return ((size_t)Tile<H, W>::PB * plane_floats<K, H, W>() + 2 * K) * sizeof(float);
+    return ((size_t)out_tile_offset<K, H, W>() +
+            (use_out_tile<T, H, W>() ? Tile<H, W>::PB * H * W : 0)) * sizeof(float);
 }
 template <int K, int H, int W>
 constexpr size_t plane_wgrad_lds_bytes() {
@@ -710,7 +742,7 @@ template <typename T, int K, int H, int W>
 int launch_plane_conv(int op, const void *src, const float *w, const float *bias, const void *taps,
                       void *dst, int N, int C, hipStream_t st) {
     constexpr int NT = Tile<H, W>::NT;
-    const size_t lds = plane_kernel_lds_bytes<K, H, W>();
+    const size_t lds = plane_kernel_lds_bytes<T, K, H, W>();
     static const int slots_f = resident_slots(plane_kernel<OP_FPROP, T, K, H, W>, NT, lds);
     static const int dbg_groups = getenv("DWO_GROUPS") ? atoi(getenv("DWO_GROUPS")) : 0;
     const int groups = dbg_groups ? dbg_groups : plane_groups(N, C, Tile<H, W>::PB, slots_f);
