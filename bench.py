@@ -53,6 +53,9 @@ def main():
                     help="repeats of the per-kernel measurement (the median is reported)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--only", default="", help="restrict the per-kernel table, e.g. 96x56:fprop")
+    ap.add_argument("--calibration-copy", action="store_true",
+                    help="also run a plain device copy of one 96x56x56 batch-64 tensor (a kernel "
+                         "of known traffic, for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build measures one GPU only (the operator has no cross-GPU "
@@ -185,12 +188,26 @@ def main():
             detail[key] = {"us": round(us, 2), "GB/s": round(gbs, 1),
                            "frac_hbm": round(gbs / HBM_PEAK_GBS, 4), "bytes": ab}
 
+    if args.calibration_copy:
+        src = sets[0][0][2]
+        dstc = torch.empty_like(src)
+        for _ in range(3):
+            dstc.copy_(src)
+        torch.cuda.synchronize()
+
+    # HBM bytes per launch of the dominant kernel from rocprofv3 FETCH_SIZE + WRITE_SIZE, each
+    # scaled by what the same counter reads for a plain copy of known size (summary and the
+    # commands under profiles/dwoconv1d_stage_sweep_f32_nchw_hbm_traffic.md); only valid for
+    # the configuration it was measured on.
+    measured_traffic = {("f32", "nchw", "roundrobin"): int((76145 + 80576) * 1024)}
+
     dom = detail.get("96x56:fprop")
     roofline = None
     if dom:
         roofline = {"bound": "hbm", "kernel": "fprop C=96 56x56 N=64 %s %s" % (args.dtype, args.layout),
                     "achieved": dom["GB/s"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                    "frac": round(dom["GB/s"] / HBM_PEAK_GBS, 4), "traffic": None,
+                    "frac": round(dom["GB/s"] / HBM_PEAK_GBS, 4),
+                    "traffic": measured_traffic.get((args.dtype, args.layout, args.theta)),
                     "launch_us": dom["us"], "algorithmic_bytes": dom["bytes"]}
 
     # ------------------------------------------------------------------ CPU baseline (oracle)

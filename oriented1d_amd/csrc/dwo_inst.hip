@@ -9,8 +9,3 @@ template int launch_plane_wgrad<DWO_INST_T, DWO_INST_K, DWO_INST_H, DWO_INST_W>(
     const void *, const void *, const void *, float *, int, int, int *, hipStream_t);
 }  // namespace dwo
 
-#ifdef DWO_DBG_TIMING
-extern "C" int dwo_dbg_read(long long *host, int n) {
-    return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(dwo::g_dbg), (size_t)n * sizeof(long long));
-}
-#endif

@@ -8,8 +8,6 @@
 // the table-driven body at the bottom (same staging, dynamic taps).
 #pragma once
 
-#include <stdlib.h>
-
 #ifndef DWO_WPE
 #define DWO_WPE 6
 #endif
@@ -109,17 +107,10 @@ constexpr int plane_floats() {
     return max_plane_floats<K, H, W>(std::make_integer_sequence<int, 8>{});
 }
 
-// scalar non-temporal store (bf16_t is a struct: store its bits)
+// scalar stores of single results (4-byte ones non-temporal, like the vector stores)
 __device__ __forceinline__ void st_out(float *p, float v) { __builtin_nontemporal_store(v, p); }
-#ifdef DWO_NT_SCALAR16
-__device__ __forceinline__ void st_out(f16_t *p, f16_t v) { __builtin_nontemporal_store(v, p); }
-__device__ __forceinline__ void st_out(bf16_t *p, bf16_t v) {
-    __builtin_nontemporal_store(v.bits, &p->bits);
-}
-#else
 __device__ __forceinline__ void st_out(f16_t *p, f16_t v) { *p = v; }
 __device__ __forceinline__ void st_out(bf16_t *p, bf16_t v) { *p = v; }
-#endif
 
 // VL consecutive activations of a plane held in registers between the global load and the LDS
 // write (VL = 4: one 16/8-byte access; VL = 1: planes whose size is not a multiple of four).
@@ -195,6 +186,28 @@ struct GeoMap {
     }
 };
 
+// Instruction-order hint for one unrolled item body of NSRC LDS reads feeding NFMA FMAs: reads
+// are issued in chunks of CH, and the FMAs that consume chunk k are placed after the reads of
+// chunk k+1, so a wave's LDS latency overlaps its own arithmetic instead of being waited out
+// chunk by chunk.
+template <int NSRC, int NFMA, int CH = 8>
+__device__ __forceinline__ void pipeline_reads_and_fmas() {
+    constexpr int NC = (NSRC + CH - 1) / CH;
+    constexpr int PER = (NFMA + NC - 1) / NC;
+    __builtin_amdgcn_sched_group_barrier(0x100, CH, 0);  // DS read
+    static_for<NC>([&](auto) {
+        __builtin_amdgcn_sched_group_barrier(0x100, CH, 0);  // next chunk's reads
+        __builtin_amdgcn_sched_group_barrier(0x002, PER, 0); // FMAs of the previous chunk
+    });
+}
+
+constexpr int plan_fma_count(const Plan &p, int L) {
+    int n = 0;
+    for (int m = 0; m < p.nsrc; m++)
+        for (int l = 0; l < L; l++) n += p.user[m][l] >= 0 ? 1 : 0;
+    return n;
+}
+
 // Workgroup -> (channel, image group).  Hardware hands consecutive workgroup ids to the eight
 // XCDs round-robin and fills the CUs of an XCD in order, while orientation (hence cost) often
 // repeats with period 8 over the channels; rotating the task id inside every aligned block of
@@ -240,6 +253,7 @@ __device__ __forceinline__ void flush_out_tile(const float *lout, T *__restrict_
         }
     }
 }
+
 
 // The two register sets of the fprop/dgrad pipeline; start() issues the loads of the first two
 // batches of images [n0, n1) of channel c.
@@ -330,6 +344,7 @@ __device__ __forceinline__ void run_canonical(const T *__restrict__ src, const f
                         if constexpr (t >= 0) acc[l] = __builtin_fmaf(v, wv[t], acc[l]);
                     });
                 });
+                pipeline_reads_and_fmas<G::plan.nsrc, plan_fma_count(G::plan, L)>();
                 if constexpr (G::CLS == CLS_H) {
                     T *o = obase + (pl * pstride + rb * W + j * L);
                     if constexpr (L == 4) {
@@ -569,6 +584,7 @@ __device__ __forceinline__ void run_canonical_wgrad(const T *__restrict__ x, con
                         if constexpr (t >= 0) acc[t] = __builtin_fmaf(v, d[l], acc[t]);
                     });
                 });
+                pipeline_reads_and_fmas<G::plan.nsrc, plan_fma_count(G::plan, L)>();
 #pragma unroll
                 for (int l = 0; l < L; l++) acc[K] += d[l];
             }
@@ -668,10 +684,6 @@ constexpr size_t plane_wgrad_lds_bytes() {
     return ((size_t)wgrad_dy_offset<K, H, W>() + Tile<H, W>::PB * H * W) * sizeof(float);
 }
 
-#ifdef DWO_DBG_TIMING
-__device__ long long g_dbg[8192 * 4];
-#endif
-
 template <int OP, typename T, int K, int H, int W>
 __global__ __launch_bounds__((Tile<H, W>::NT)) __attribute__((amdgpu_waves_per_eu(DWO_WPE, 8))) void plane_kernel(
     const T *__restrict__ src, const float *__restrict__ wt, const float *__restrict__ bias,
@@ -681,9 +693,6 @@ __global__ __launch_bounds__((Tile<H, W>::NT)) __attribute__((amdgpu_waves_per_e
     plane_task(C, groups, c, group);
     int n0, n1;
     group_range<Tile<H, W>::PB>(N, groups, group, n0, n1);
-#ifdef DWO_DBG_TIMING
-    const long long t_start = wall_clock64();
-#endif
     ConvStagers<T, H, W> sg;
     sg.start(src, c, C, n0, n1);  // HBM latency overlaps the class lookup, weights and zero fill
     const int cls = taps_class(blob, C, K)[c];
@@ -704,23 +713,6 @@ __global__ __launch_bounds__((Tile<H, W>::NT)) __attribute__((amdgpu_waves_per_e
             run_table<OP, T, K, H, W>(src, wt, bias, taps_dhdw(blob), dst, lds, c, C, n0, n1, sg);
     }
 #undef DWO_CASE
-#ifdef DWO_DBG_TIMING
-    if ((threadIdx.x & 63) == 0 && blockIdx.x < 1024) {
-        unsigned hwid;
-        asm volatile("s_getreg_b32 %0, hwreg(HW_REG_HW_ID)" : "=s"(hwid));
-        g_dbg[8192 * 2 + blockIdx.x * 8 + (threadIdx.x >> 6)] = hwid;
-    }
-    if (threadIdx.x == 0 && blockIdx.x < 4096) {
-        unsigned hwid;
-        asm volatile("s_getreg_b32 %0, hwreg(HW_REG_HW_ID)" : "=s"(hwid));
-        unsigned xcc;
-        asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
-        g_dbg[blockIdx.x * 4 + 0] = t_start;
-        g_dbg[blockIdx.x * 4 + 1] = wall_clock64();
-        g_dbg[blockIdx.x * 4 + 2] = ((long long)xcc << 32) | hwid;
-        g_dbg[blockIdx.x * 4 + 3] = ((long long)cls << 32) | (unsigned)(n1 - n0);
-    }
-#endif
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -744,8 +736,7 @@ int launch_plane_conv(int op, const void *src, const float *w, const float *bias
     constexpr int NT = Tile<H, W>::NT;
     const size_t lds = plane_kernel_lds_bytes<T, K, H, W>();
     static const int slots_f = resident_slots(plane_kernel<OP_FPROP, T, K, H, W>, NT, lds);
-    static const int dbg_groups = getenv("DWO_GROUPS") ? atoi(getenv("DWO_GROUPS")) : 0;
-    const int groups = dbg_groups ? dbg_groups : plane_groups(N, C, Tile<H, W>::PB, slots_f);
+    const int groups = plane_groups(N, C, Tile<H, W>::PB, slots_f);
     const dim3 grid(C * groups), block(NT);
     if (op == OP_FPROP)
         plane_kernel<OP_FPROP, T, K, H, W><<<grid, block, lds, st>>>((const T *)src, w, bias, taps,
