@@ -53,6 +53,8 @@ def main():
                     help="repeats of the per-kernel measurement (the median is reported)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--only", default="", help="restrict the per-kernel table, e.g. 96x56:fprop")
+    ap.add_argument("--model-iters", type=int, default=5,
+                    help="timed ConvNeXt-T-1D inference forwards (batch 128, bf16); 0 skips it")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="also run a plain device copy of one 96x56x56 batch-64 tensor (a kernel "
                          "of known traffic, for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE)")
@@ -237,6 +239,67 @@ def main():
                          "(%.1f s)" % cpu_s,
                "host_cpus": os.cpu_count()}
 
+    # ------------------------------------------------------------------ ConvNeXt-T-1D images/s
+    # Second half of the metric: inference forward of the harness (random-init weights, bf16,
+    # batch 128 of 3x224x224 N(0,1) images, 1000 classes); its CPU counterpart (same harness on
+    # the host, fp32, batch 8, oriented convs by the oracle) is reported beside it.
+    model_info = None
+    if args.model_iters > 0:
+        del sets, calls, keep
+        torch.cuda.empty_cache()
+        from oriented1d_amd.convnext1d import convnext_tiny_1d
+        from oriented1d_amd.dwoconv1d import DepthwiseOrientedConv1d
+
+        torch.manual_seed(0)
+        model = convnext_tiny_1d(variant="1d").to(dev).to(torch.bfloat16).eval()
+        imgs = torch.randn(128, 3, 224, 224, device=dev).to(torch.bfloat16)
+        with torch.no_grad():
+            for _ in range(2):
+                model(imgs)
+            torch.cuda.synchronize()
+            m0 = time.perf_counter()
+            for _ in range(args.model_iters):
+                model(imgs)
+            torch.cuda.synchronize()
+            m1 = time.perf_counter()
+        gpu_ips = 128 * args.model_iters / (m1 - m0)
+        model_info = {"model": "ConvNeXt-T-1D inference, random init, bf16, batch 128, 3x224x224",
+                      "images_per_s": round(gpu_ips, 1),
+                      "ms_per_batch": round((m1 - m0) * 1e3 / args.model_iters, 2)}
+        if not args.no_cpu_baseline:
+            from oracle import dwo_oracle as oracle
+
+            cpu_model = convnext_tiny_1d(variant="1d").eval()
+            nthreads = oracle.max_threads()
+
+            def host_conv(mod):
+                def fwd(t):
+                    o = oracle.module_forward(
+                        t.numpy(), mod.weight.detach().numpy(), mod.theta.detach().numpy(),
+                        bias=mod.bias.detach().numpy(), stride=mod.stride[0], nhwc=mod.nhwc,
+                        resid=mod.resid is not None, acc="f32")
+                    return torch.from_numpy(o)
+                return fwd
+
+            # threads only affects the C loops' channel partition (bit-identical results)
+            _fprop = oracle.fprop
+            oracle.fprop = lambda *a, **k: _fprop(*a, **{**k, "threads": nthreads})
+            for mod in cpu_model.modules():
+                if isinstance(mod, DepthwiseOrientedConv1d):
+                    mod.forward = host_conv(mod)
+            cimgs = torch.randn(8, 3, 224, 224)
+            with torch.no_grad():
+                cpu_model(cimgs)
+                c0 = time.perf_counter()
+                for _ in range(3):
+                    cpu_model(cimgs)
+                c1 = time.perf_counter()
+            oracle.fprop = _fprop
+            model_info["cpu_images_per_s"] = round(8 * 3 / (c1 - c0), 2)
+            model_info["cpu_config"] = ("same harness on the host: fp32, batch 8, 3 forwards, torch "
+                                        "CPU ops with %d threads, oriented convs by the oracle's "
+                                        "loops on %d threads" % (torch.get_num_threads(), nthreads))
+
     out = {
         "metric": "dwoconv1d fprop/dgrad/wgrad GB/s (% HBM peak); ConvNeXt-T-1D img/s",
         "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
@@ -249,6 +312,7 @@ def main():
                    "algorithmic_bytes_per_step": step_bytes},
         "frac_hbm_peak": round(value / HBM_PEAK_GBS, 4),
         "detail": detail, "roofline": roofline, "cpu_baseline": cpu,
+        "convnext_t_1d": model_info,
     }
     print(json.dumps(out))
 

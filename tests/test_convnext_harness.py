@@ -1,0 +1,92 @@
+"""ConvNeXt-1D / 1D++ harness: structural known answers on CPU (parameter counts published in
+the reference's README.md:41-46, state_dict naming of models/convnext.py) and, on the GPU, the
+whole network against the same network with every oriented conv computed by the CPU oracle."""
+import numpy as np
+import pytest
+import torch
+
+from oriented1d_amd.convnext1d import (ConvNeXt1D, channel_angles, convnext_base_1d,
+                                       convnext_tiny_1d)
+from oriented1d_amd.dwoconv1d import DepthwiseOrientedConv1d
+
+
+@pytest.mark.parametrize("factory,variant,millions", [
+    (convnext_tiny_1d, "1d", 28.5), (convnext_tiny_1d, "1dpp", 29.2),
+    (convnext_base_1d, "1d", 88.0), (convnext_base_1d, "1dpp", 90.0)])
+def test_parameter_counts_match_published(factory, variant, millions):
+    n = sum(p.numel() for p in factory(variant=variant).parameters())
+    assert abs(n / 1e6 - millions) < 0.45, n
+
+
+def test_state_dict_layout_and_angles():
+    m = convnext_tiny_1d(variant="1dpp")
+    sd = m.state_dict()
+    for key in ("downsample_layers.0.pw1.weight", "downsample_layers.0.dw1.theta",
+                "downsample_layers.0.norm3.bias", "downsample_layers.1.0.weight",
+                "downsample_layers.1.1.weight", "stages.0.0.dwconv1.weight",
+                "stages.0.0.dwconv2.theta", "stages.2.8.pwconv2.bias", "stages.3.2.gamma",
+                "norm.weight", "head.bias"):
+        assert key in sd, key
+    assert tuple(sd["stages.0.0.dwconv1.weight"].shape) == (96, 1, 1, 15)
+    assert tuple(sd["stages.0.0.dwconv2.weight"].shape) == (384, 1, 1, 31)
+    assert tuple(sd["downsample_layers.0.dw1.weight"].shape) == (64, 1, 1, 15)
+    m1 = convnext_tiny_1d(variant="1d")
+    assert "stages.1.1.dwconv.bias" in m1.state_dict()
+    assert tuple(m1.state_dict()["downsample_layers.0.dw2.weight"].shape) == (64, 1, 1, 31)
+    # contiguous groups of C/8 channels per direction; +90 degrees on odd layers
+    a = channel_angles(96)
+    assert a[0] == 0.0 and a[11] == 0.0 and abs(a[12] - np.pi / 8) < 1e-12 and abs(a[95] - 7 * np.pi / 8) < 1e-12
+    th0, th1 = m1.stages[0][0].dwconv.theta, m1.stages[0][1].dwconv.theta
+    assert torch.allclose((th0 + np.pi / 2) % np.pi, th1 % np.pi, atol=1e-6)
+    assert m1.stages[0][0].dwconv.nhwc is False and m.stages[0][0].dwconv2.nhwc is True
+    assert m.stages[0][0].dwconv2.resid is not None and m.downsample_layers[0].dw1.stride == (2, 2)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("variant", ["1d", "1dpp"])
+def test_network_matches_oracle_composition(oracle, variant):
+    torch.manual_seed(0)
+    m = ConvNeXt1D(depths=(1, 2, 1, 1), dims=(16, 32, 64, 128), variant=variant, stem_dim1=24,
+                   num_classes=10, layer_scale_init_value=1.0).cuda().eval()
+    for name, p in m.named_parameters():  # biases away from their zero defaults
+        if name.endswith("bias"):
+            torch.nn.init.normal_(p, std=0.1)
+    x = torch.randn(2, 3, 64, 64, device="cuda")
+    with torch.no_grad():
+        y = m(x)
+
+    def oracle_forward(mod):
+        def fwd(t):
+            w = mod.weight.detach().float().cpu().numpy()
+            b = mod.bias.detach().float().cpu().numpy()
+            th = mod.theta.detach().float().cpu().numpy()
+            out = oracle.module_forward(t.detach().float().cpu().numpy(), w, th, bias=b,
+                                        stride=mod.stride[0], nhwc=mod.nhwc,
+                                        resid=mod.resid is not None)
+            return torch.from_numpy(out).to(device=t.device, dtype=t.dtype)
+        return fwd
+
+    for mod in m.modules():
+        if isinstance(mod, DepthwiseOrientedConv1d):
+            mod.forward = oracle_forward(mod)
+    with torch.no_grad():
+        y_ref = m(x)
+    err = (y - y_ref).abs().max().item() / y_ref.abs().max().item()
+    assert y.shape == (2, 10) and err < 2e-5, err
+
+
+@pytest.mark.gpu
+def test_training_step_and_stage_outputs():
+    torch.manual_seed(1)
+    m = ConvNeXt1D(depths=(1, 1, 1, 1), dims=(16, 32, 64, 128), variant="1dpp", stem_dim1=16,
+                   out_stages=True, drop_path_rate=0.2).cuda().train()
+    x = torch.randn(2, 3, 64, 64, device="cuda")
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        outs = m(x)
+    assert [tuple(o.shape[1:]) for o in outs] == [(16, 16, 16), (32, 8, 8), (64, 4, 4), (128, 2, 2)]
+    sum(o.float().square().mean() for o in outs).backward()
+    for name, p in m.named_parameters():
+        if name.endswith("theta"):
+            assert p.grad is None, name
+        else:
+            assert p.grad is not None and torch.isfinite(p.grad).all(), name
