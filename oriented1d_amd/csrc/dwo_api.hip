@@ -6,6 +6,7 @@
 
 #include "dwo_common.h"
 #include "dwo_generic.h"
+#include "dwo_nhwc.h"
 #include "dwo_dispatch.h"
 
 using namespace dwo;
@@ -91,14 +92,62 @@ int try_plane_wgrad(const void *x, const void *dy, const void *taps, float *part
     return -100;
 }
 
+// NHWC with a kernel size that has lane-resident tap kernels; -100 otherwise
+#define DWO_NHWC_KS(X) X(7) X(13) X(15) X(27) X(31)
+bool nhwc_has_k(int K) {
+#define DWO_MATCH(K_) if (K == K_) return true;
+    DWO_NHWC_KS(DWO_MATCH)
+#undef DWO_MATCH
+    return false;
+}
+
 // wgrad partial-sum count per (channel, tap): an upper bound that sizes the scratch buffer
 // (the staged path picks its group count from the device's occupancy at launch, never more
 // than kMaxPlaneGroups nor than the number of staged batches).
 int wgrad_max_partials(const ConvDims &d, int layout) {
     const int PB = plane_batch(d, layout);
+    if (PB == 0 && layout == DWO_NHWC && nhwc_has_k(d.K)) {
+        int ppw = 0;
+        return nhwc_wgrad_groups((long)d.N * d.P * d.Q, (d.C + 63) / 64, &ppw);
+    }
     if (PB == 0) return wgrad_generic_split(d, layout).G;
     const int nbatch = (d.N + PB - 1) / PB;
     return nbatch < kMaxPlaneGroups ? nbatch : kMaxPlaneGroups;
+}
+
+template <typename T, int MODE>
+int try_nhwc_conv(const void *src, const float *w, const float *bias, const void *taps, void *dst,
+                  const ConvDims &d, int layout, hipStream_t st) {
+    if (layout != DWO_NHWC || !nhwc_has_k(d.K)) return -100;
+    if (MODE == NHWC_DGRAD && d.stride != 1) return -100;  // strided dgrad: generic kernel
+    const int slabs = (d.C + 63) / 64;
+    const long per_image = MODE == NHWC_DGRAD ? (long)d.H * d.W : (long)d.P * d.Q;
+    const int ppw = nhwc_pix_per_wave(d.N * per_image, slabs);
+    const dim3 grid(nhwc_conv_grid(d.N, per_image, ppw, slabs)), block(kNhwcThreads);
+#define DWO_MATCH(K_)                                                                         \
+    if (d.K == K_)                                                                            \
+        nhwc_conv_kernel<T, K_, MODE><<<grid, block, 0, st>>>((const T *)src, w, bias,        \
+                                                              taps_dhdw(taps), (T *)dst, d, ppw);
+    DWO_NHWC_KS(DWO_MATCH)
+#undef DWO_MATCH
+    return launch_status();
+}
+
+template <typename T>
+int try_nhwc_wgrad(const void *dy, const void *x, const void *taps, float *part, int *groups,
+                   const ConvDims &d, hipStream_t st) {
+    const int slabs = (d.C + 63) / 64;
+    int ppw = 0;
+    const int NG = nhwc_wgrad_groups((long)d.N * d.P * d.Q, slabs, &ppw);
+    *groups = NG;
+    const dim3 grid(slabs, NG), block(kNhwcThreads);
+#define DWO_MATCH(K_)                                                                          \
+    if (d.K == K_)                                                                             \
+        nhwc_wgrad_kernel<T, K_><<<grid, block, 0, st>>>((const T *)dy, (const T *)x,          \
+                                                         taps_dhdw(taps), part, d, ppw, NG);
+    DWO_NHWC_KS(DWO_MATCH)
+#undef DWO_MATCH
+    return launch_status();
 }
 
 template <typename T>
@@ -106,6 +155,8 @@ int fprop_t(const void *x, const float *w, const float *bias, const void *taps, 
             const ConvDims &d, int layout, hipStream_t st) {
     const int fast = try_plane_conv<T>(OP_FPROP, x, w, bias, taps, y, d, layout, st);
     if (fast != -100) return fast;
+    const int nhwc = try_nhwc_conv<T, NHWC_FPROP>(x, w, bias, taps, y, d, layout, st);
+    if (nhwc != -100) return nhwc;
     const int total = d.N * d.C * d.P * d.Q;
     const dim3 grid((total + 255) / 256), block(256);
     const int8_t *tp = taps_dhdw(taps);
@@ -123,6 +174,8 @@ int dgrad_t(const void *dy, const float *w, const void *taps, void *dx, const Co
             int layout, hipStream_t st) {
     const int fast = try_plane_conv<T>(OP_DGRAD, dy, w, nullptr, taps, dx, d, layout, st);
     if (fast != -100) return fast;
+    const int nhwc = try_nhwc_conv<T, NHWC_DGRAD>(dy, w, nullptr, taps, dx, d, layout, st);
+    if (nhwc != -100) return nhwc;
     const int total = d.N * d.C * d.H * d.W;
     const dim3 grid((total + 255) / 256), block(256);
     const int8_t *tp = taps_dhdw(taps);
@@ -142,6 +195,8 @@ int wgrad_t(const void *dy, const void *x, const void *taps, float *dw, float *d
     int rc, NG = 0;
     if (plane_batch(d, layout) != 0) {
         rc = try_plane_wgrad<T>(x, dy, taps, part, &NG, d, st);
+    } else if (layout == DWO_NHWC && nhwc_has_k(d.K)) {
+        rc = try_nhwc_wgrad<T>(dy, x, taps, part, &NG, d, st);
     } else {
         const WgradSplit s = wgrad_generic_split(d, layout);
         NG = s.G;
