@@ -97,6 +97,86 @@ constexpr Plan make_plan(int o, int K, int L, int H, int W) {
     return p;
 }
 
+
+// Pair plan, for 16-bit activations.  LDS then holds, at every position, the 32-bit word
+// (x[pos], x[pos + e]) -- the element and its neighbour along the step direction -- so one read
+// feeds two taps of a run through a dot2 instruction (two multiply-adds into an fp32
+// accumulator).  Each run of taps t0, t0+e, t0+2e, ... is cut into pairs from its start;
+// pair k of a run, for output l, is the word at t0 + (2k + l) * e.
+struct PairPlan {
+    int nsrc = 0;                      // distinct word positions per item
+    int npair = 0;                     // distinct (tap, next tap) weight pairs
+    int16_t sh[kMaxSrc] = {};
+    int16_t sw[kMaxSrc] = {};
+    int8_t user[kMaxSrc][kMaxL] = {};  // weight pair feeding output l, or -1
+    int8_t pair_lo[64] = {};           // representative taps of a weight pair (hi may be -1)
+    int8_t pair_hi[64] = {};
+    int8_t rep[64] = {};
+    int hmin = 0, hmax = 0, wmin = 0, wmax = 0;  // box of the words read and of the neighbours
+                                                 // written while staging
+};
+
+constexpr PairPlan make_pair_plan(int o, int K, int L, int H, int W) {
+    PairPlan p{};
+    const int eh = step_h(o), ew = step_w(o);
+    constexpr int G = 48, GS = 2 * G + 1;
+    int8_t grid[GS][GS] = {};
+    int16_t src[GS][GS] = {};
+    for (int i = 0; i < GS; i++)
+        for (int j = 0; j < GS; j++) grid[i][j] = -1, src[i][j] = -1;
+    for (int s = 0; s < K; s++) {
+        const int dh = canon_dh(o, K, s), dw = canon_dw(o, K, s);
+        p.rep[s] = -1;
+        if (dh >= H || dh <= -H || dw >= W || dw <= -W) continue;
+        if (grid[dh + G][dw + G] < 0) grid[dh + G][dw + G] = (int8_t)s;
+        p.rep[s] = grid[dh + G][dw + G];
+    }
+    // staging writes x[pos] into the words at pos and pos - e of every interior position
+    p.hmin = eh > 0 ? -1 : 0, p.hmax = eh < 0 ? 1 : 0, p.wmin = ew > 0 ? -1 : 0, p.wmax = 0;
+    for (int h = -G + 1; h < G; h++)
+        for (int w = -G + 1; w < G; w++) {
+            if (grid[h + G][w + G] < 0) continue;
+            const int ph = h - eh + G, pw = w - ew + G;
+            if (ph >= 0 && ph < GS && pw >= 0 && pw < GS && grid[ph][pw] >= 0) continue;  // not a run start
+            // walk the run from (h, w)
+            int ch = h, cw = w;
+            while (ch + G < GS && cw + G < GS && ch + G >= 0 && cw + G >= 0 && grid[ch + G][cw + G] >= 0) {
+                const int lo = grid[ch + G][cw + G];
+                const int nh = ch + eh, nw = cw + ew;
+                const bool has = nh + G < GS && nw + G < GS && nh + G >= 0 && nw + G >= 0 &&
+                                 grid[nh + G][nw + G] >= 0;
+                const int hi = has ? grid[nh + G][nw + G] : -1;
+                const int pid = p.npair++;
+                p.pair_lo[pid] = (int8_t)lo;
+                p.pair_hi[pid] = (int8_t)hi;
+                for (int l = 0; l < L; l++) {
+                    const int sh = ch + l * eh, sw = cw + l * ew;
+                    if (src[sh + G][sw + G] < 0) {
+                        src[sh + G][sw + G] = (int16_t)p.nsrc;
+                        p.sh[p.nsrc] = (int16_t)sh;
+                        p.sw[p.nsrc] = (int16_t)sw;
+                        for (int q = 0; q < kMaxL; q++) p.user[p.nsrc][q] = -1;
+                        p.nsrc++;
+                    }
+                    p.user[src[sh + G][sw + G]][l] = (int8_t)pid;
+                    if (sh < p.hmin) p.hmin = sh;
+                    if (sh > p.hmax) p.hmax = sh;
+                    if (sw < p.wmin) p.wmin = sw;
+                    if (sw > p.wmax) p.wmax = sw;
+                }
+                ch += 2 * eh, cw += 2 * ew;
+                if (!has) break;
+            }
+        }
+    return p;
+}
+constexpr int pair_plan_dot_count(const PairPlan &p, int L) {
+    int n = 0;
+    for (int m = 0; m < p.nsrc; m++)
+        for (int l = 0; l < L; l++) n += p.user[m][l] >= 0 ? 1 : 0;
+    return n;
+}
+
 constexpr int round_up(int v, int m) { return (v + m - 1) / m * m; }
 constexpr int cmax(int a, int b) { return a > b ? a : b; }
 
@@ -109,13 +189,25 @@ constexpr int bank_stride(int need, int mult, int target) {
     return need | 1;
 }
 
-// LDS geometry of one (orientation, K, L, H, W) variant.  All sizes in floats.
-template <int O, int K, int L, int H, int W>
+template <bool PAIR>
+struct PlanFor {
+    static constexpr Plan make(int o, int K, int L, int H, int W) { return make_plan(o, K, L, H, W); }
+};
+template <>
+struct PlanFor<true> {
+    static constexpr PairPlan make(int o, int K, int L, int H, int W) {
+        return make_pair_plan(o, K, L, H, W);
+    }
+};
+
+// LDS geometry of one (orientation, K, L, H, W) variant.  All sizes in 32-bit words (floats, or
+// element pairs when PAIR).
+template <int O, int K, int L, int H, int W, bool PAIR = false>
 struct Geo {
     static constexpr int CLS = orient_class(O);
     static constexpr int L_ = L;
     static constexpr int EH = step_h(O), EW = step_w(O);
-    static constexpr Plan plan = make_plan(O, K, L, H, W);
+    static constexpr auto plan = PlanFor<PAIR>::make(O, K, L, H, W);
 
     static constexpr int LR = CLS == CLS_H ? 1 : L;              // rows per row-block
     static constexpr int RB = (H + LR - 1) / LR;                 // row-blocks per plane
@@ -164,16 +256,28 @@ struct Tile<56, 56> {  // 784 / 448 / 448 items per plane
     static constexpr int LH = 4, LV = 7, LD = 8, PB = 1, NT = 448;
 };
 template <>
+#ifndef DWO_NTS
+#define DWO_NTS 448
+#endif
+#ifndef DWO_PB28
+#define DWO_PB28 2
+#endif
+#ifndef DWO_PB14
+#define DWO_PB14 4
+#endif
+#ifndef DWO_PB7
+#define DWO_PB7 8
+#endif
 struct Tile<28, 28> {  // 196 / 196 / 224
-    static constexpr int LH = 4, LV = 4, LD = 4, PB = 2, NT = 448;
+    static constexpr int LH = 4, LV = 4, LD = 4, PB = DWO_PB28, NT = DWO_NTS;
 };
 template <>
 struct Tile<14, 14> {  // 98 / 98 / 112
-    static constexpr int LH = 2, LV = 2, LD = 2, PB = 4, NT = 448;
+    static constexpr int LH = 2, LV = 2, LD = 2, PB = DWO_PB14, NT = DWO_NTS;
 };
 template <>
 struct Tile<7, 7> {  // 49 / 49 / 56
-    static constexpr int LH = 1, LV = 1, LD = 1, PB = 8, NT = 448;
+    static constexpr int LH = 1, LV = 1, LD = 1, PB = DWO_PB7, NT = DWO_NTS;
 };
 template <int H, int W>
 constexpr int tile_L(int o) {

@@ -50,6 +50,7 @@ struct Vec4<float> {
         __builtin_nontemporal_store(v, reinterpret_cast<f4 *>(p));
     }
     __device__ __forceinline__ float get(int i) const { return v[i]; }
+    __device__ __forceinline__ uint16_t bits(int) const { return 0; }
     __device__ __forceinline__ void set(float a, float b, float c, float d) {
         v[0] = a, v[1] = b, v[2] = c, v[3] = d;
     }
@@ -68,6 +69,9 @@ struct Vec4<bf16_t> {
         const uint32_t w = i < 2 ? v.x : v.y;
         return __uint_as_float((i & 1) ? (w & 0xffff0000u) : (w << 16));
     }
+    __device__ __forceinline__ uint16_t bits(int i) const {
+        return (uint16_t)((i < 2 ? v.x : v.y) >> (16 * (i & 1)));
+    }
     __device__ __forceinline__ void set(float a, float b, float c, float d) {
         v.x = (uint32_t)from_float<bf16_t>(a).bits | ((uint32_t)from_float<bf16_t>(b).bits << 16);
         v.y = (uint32_t)from_float<bf16_t>(c).bits | ((uint32_t)from_float<bf16_t>(d).bits << 16);
@@ -84,6 +88,9 @@ struct Vec4<f16_t> {
         __builtin_nontemporal_store(v, reinterpret_cast<h4 *>(p));
     }
     __device__ __forceinline__ float get(int i) const { return (float)v[i]; }
+    __device__ __forceinline__ uint16_t bits(int i) const {
+        return __builtin_bit_cast(uint16_t, (_Float16)v[i]);
+    }
     __device__ __forceinline__ void set(float a, float b, float c, float d) {
         v[0] = (_Float16)a, v[1] = (_Float16)b, v[2] = (_Float16)c, v[3] = (_Float16)d;
     }
@@ -100,6 +107,7 @@ constexpr int max_plane_floats(std::integer_sequence<int, Os...>) {
     constexpr int PAD = table_pad<K, H, W>();
     int m = (H + 2 * PAD) * (W + 2 * PAD + 3);  // table-driven body
     ((m = cmax(m, Geo<Os, K, tile_L<H, W>(Os), H, W>::PLANE)), ...);
+    ((m = cmax(m, Geo<Os, K, tile_L<H, W>(Os), H, W, true>::PLANE)), ...);
     return m;
 }
 template <int K, int H, int W>
@@ -112,6 +120,22 @@ __device__ __forceinline__ void st_out(float *p, float v) { __builtin_nontempora
 __device__ __forceinline__ void st_out(f16_t *p, f16_t v) { *p = v; }
 __device__ __forceinline__ void st_out(bf16_t *p, bf16_t v) { *p = v; }
 
+// 16-bit patterns of the 16-bit element types, and the two-element dot product with fp32
+// accumulation they feed (a and b each hold two elements; c + a.lo*b.lo + a.hi*b.hi).
+__device__ __forceinline__ uint16_t raw16(bf16_t v) { return v.bits; }
+__device__ __forceinline__ uint16_t raw16(f16_t v) { return __builtin_bit_cast(uint16_t, v); }
+__device__ __forceinline__ uint16_t raw16(float) { return 0; }
+__device__ __forceinline__ float dot2_acc(unsigned a, unsigned b, float c, bf16_t) {
+    typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
+    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf2, a), __builtin_bit_cast(bf2, b), c,
+                                           false);
+}
+__device__ __forceinline__ float dot2_acc(unsigned a, unsigned b, float c, f16_t) {
+    typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+    return __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, a), __builtin_bit_cast(h2, b), c, false);
+}
+__device__ __forceinline__ float dot2_acc(unsigned, unsigned, float c, float) { return c; }
+
 // VL consecutive activations of a plane held in registers between the global load and the LDS
 // write (VL = 4: one 16/8-byte access; VL = 1: planes whose size is not a multiple of four).
 template <typename T, int VL>
@@ -123,6 +147,7 @@ struct Chunk<T, 1> {
     T v;
     __device__ __forceinline__ void load(const T *p) { v = *p; }
     __device__ __forceinline__ float get(int) const { return to_float(v); }
+    __device__ __forceinline__ uint16_t bits(int) const { return raw16(v); }
 };
 
 // Staging of PB planes (n, c), n = nb .. nb+PB-1, through registers into LDS.  `Map` gives the
@@ -170,19 +195,69 @@ struct Stager {
             }
         }
     }
+    // Pair staging for 16-bit activations: element (r, w) becomes the low half of the word at
+    // (r, w) and the high half of the word at (r - EH, w - EW), so that every word holds an
+    // element and its neighbour along the step direction (EH, EW).
+    template <class Map, int PLS, int EH, int EW>
+    __device__ __forceinline__ void commit_pairs(float *lds, int nvalid) const {
+        uint16_t *half = reinterpret_cast<uint16_t *>(lds);
+#pragma unroll
+        for (int k = 0; k < PF; k++) {
+            const unsigned f = threadIdx.x + k * NT;
+            const unsigned pl = f / FP, g = f % FP;
+            if (f < PB * FP && (int)pl < nvalid) {
+                if constexpr (W % VL == 0) {
+                    // one address per chunk; every half-word sits at a constant distance from it
+                    const unsigned r = g / (W / VL), w0 = (g % (W / VL)) * VL;
+                    uint16_t *q = half + 2 * (pl * PLS + Map::index((int)r, (int)w0));
+                    if constexpr (EH == 0 && EW == 1 && VL == 4) {
+                        // a chunk holds both halves of its first three words
+                        unsigned *q32 = reinterpret_cast<unsigned *>(q);
+#pragma unroll
+                        for (int e = 0; e < 3; e++)
+                            q32[Map::step(e)] =
+                                (unsigned)pre[k].bits(e) | (unsigned)pre[k].bits(e + 1) << 16;
+                        q[2 * Map::step(3)] = pre[k].bits(3);
+                        q[2 * Map::pair_step(0) + 1] = pre[k].bits(0);
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < VL; e++) {
+                            const uint16_t v = pre[k].bits(e);
+                            q[2 * Map::step(e)] = v;
+                            q[2 * Map::pair_step(e) + 1] = v;
+                        }
+                    }
+                } else {
+#pragma unroll
+                    for (int e = 0; e < VL; e++) {
+                        const unsigned i = g * VL + e;
+                        const unsigned r = i / W, w = i % W;
+                        const uint16_t v = pre[k].bits(e);
+                        half[2 * (pl * PLS + Map::index((int)r, (int)w))] = v;
+                        half[2 * (pl * PLS + Map::index((int)r - EH, (int)w - EW)) + 1] = v;
+                    }
+                }
+            }
+        }
+    }
 };
 
 // Interior-element map of a canonical geometry.  step(e) is the LDS distance from element
 // (r, w0) to (r, w0 + e) when w0 is a multiple of four and the row is at least four wide.
 template <class G>
 struct GeoMap {
-    static __device__ __forceinline__ unsigned index(unsigned r, unsigned w) {
+    static __device__ __forceinline__ unsigned index(int r, int w) {
         return G::interior_row(r) + G::col(w + G::PL);
     }
     static constexpr int step(int e) {
         return G::CLS == CLS_H ? (G::L_ >= 4 ? (e % G::L_) * G::SUB + e / G::L_
                                              : G::col(e + G::PL) - G::col(G::PL))
                                : e;
+    }
+    // distance from (r, w0) to the position one step (EH, EW) before (r, w0 + e)
+    static constexpr int pair_step(int e) {
+        return G::CLS == CLS_H ? (e > 0 ? step(e - 1) : (G::L_ - 1) * G::SUB - 1)
+                               : e - G::EH * G::RS - G::EW;
     }
 };
 
@@ -201,7 +276,8 @@ __device__ __forceinline__ void pipeline_reads_and_fmas() {
     });
 }
 
-constexpr int plan_fma_count(const Plan &p, int L) {
+template <class P>
+constexpr int plan_fma_count(const P &p, int L) {
     int n = 0;
     for (int m = 0; m < p.nsrc; m++)
         for (int l = 0; l < L; l++) n += p.user[m][l] >= 0 ? 1 : 0;
@@ -272,6 +348,19 @@ struct ConvStagers {
 // ---------------------------------------------------------------------------------------------
 // canonical body
 // ---------------------------------------------------------------------------------------------
+// 16-bit activations take the pair form: LDS words hold (x[pos], x[pos + e]) in the activation's
+// own format, weights are rounded to that format and packed two taps to a word, and one dot2
+// replaces two FMAs (accumulation stays fp32).
+// Used where it measures faster: orientations whose step runs along a row (there most staged
+// words leave a thread as whole 32-bit writes) on planes whose rows split into 4-element chunks.
+template <typename T, int O, int W>
+constexpr bool use_pairs() {
+#ifdef DWO_NO_PAIRS
+    return false;
+#else
+    return sizeof(T) == 2 && orient_class(O) == CLS_H && W % 4 == 0;
+#endif
+}
 template <int O, int OP, typename T, int K, int H, int W>
 __device__ __forceinline__ void run_canonical(const T *__restrict__ src, const float *__restrict__ wt,
                                               const float *__restrict__ bias, T *__restrict__ dst,
@@ -279,7 +368,8 @@ __device__ __forceinline__ void run_canonical(const T *__restrict__ src, const f
                                               ConvStagers<T, H, W> &sg) {
     constexpr int L = tile_L<H, W>(O);
     constexpr int PB = Tile<H, W>::PB, NT = Tile<H, W>::NT;
-    using G = Geo<O, K, L, H, W>;
+    constexpr bool PAIR = use_pairs<T, O, W>();
+    using G = Geo<O, K, L, H, W, PAIR>;
     constexpr int PLS = plane_floats<K, H, W>();  // LDS plane stride (same for all orientations)
     constexpr int ITERS = (PB * G::IPP + NT - 1) / NT;
     const unsigned tid = threadIdx.x;
@@ -303,6 +393,20 @@ __device__ __forceinline__ void run_canonical(const T *__restrict__ src, const f
         }
     });
     const float bv = (OP == OP_FPROP && bias != nullptr) ? bias[c] : 0.f;
+    // pair form: (tap, next tap along the run) as two 16-bit weights per uniform word
+    constexpr int NPAIR = [] {
+        if constexpr (PAIR) return cmax((int)G::plan.npair, 1);
+        else return 1;
+    }();
+    unsigned wp[NPAIR];
+    if constexpr (PAIR) {
+        static_for<NPAIR>([&](auto q) {
+            constexpr int lo = G::plan.pair_lo[q], hi = G::plan.pair_hi[q];
+            unsigned v = raw16(from_float<T>(wv[lo]));
+            if constexpr (hi >= 0) v |= (unsigned)raw16(from_float<T>(wv[hi])) << 16;
+            wp[q] = __builtin_amdgcn_readfirstlane(v);
+        });
+    }
 
     // zero the staging area once; interiors are overwritten per batch, halos stay zero
     for (unsigned i = tid; i < PB * PLS; i += NT) lds[i] = 0.f;
@@ -321,7 +425,10 @@ __device__ __forceinline__ void run_canonical(const T *__restrict__ src, const f
             if (nb > n0)
                 flush_out_tile<T, H, W, PB, NT>(lout, dbase + (size_t)(nb - PB) * pstride, pstride, PB);
         }
-        stg.template commit<GeoMap<G>, PLS>(lds, nvalid);
+        if constexpr (PAIR)
+            stg.template commit_pairs<GeoMap<G>, PLS, G::EH, G::EW>(lds, nvalid);
+        else
+            stg.template commit<GeoMap<G>, PLS>(lds, nvalid);
         __syncthreads();
         if (nb + 2 * PB < n1)
             stg.prefetch(sbase + (size_t)(nb + 2 * PB) * pstride, pstride, n1 - nb - 2 * PB);
@@ -338,11 +445,19 @@ __device__ __forceinline__ void run_canonical(const T *__restrict__ src, const f
                 for (int l = 0; l < L; l++) acc[l] = bv;
                 static_for<G::plan.nsrc>([&](auto m) {
                     constexpr int off = G::imm(G::plan.sh[m], G::plan.sw[m]);
-                    const float v = base[off];
-                    static_for<L>([&](auto l) {
-                        constexpr int t = G::plan.user[m][l];
-                        if constexpr (t >= 0) acc[l] = __builtin_fmaf(v, wv[t], acc[l]);
-                    });
+                    if constexpr (PAIR) {
+                        const unsigned v = reinterpret_cast<const unsigned *>(base)[off];
+                        static_for<L>([&](auto l) {
+                            constexpr int q = G::plan.user[m][l];
+                            if constexpr (q >= 0) acc[l] = dot2_acc(v, wp[q], acc[l], T{});
+                        });
+                    } else {
+                        const float v = base[off];
+                        static_for<L>([&](auto l) {
+                            constexpr int t = G::plan.user[m][l];
+                            if constexpr (t >= 0) acc[l] = __builtin_fmaf(v, wv[t], acc[l]);
+                        });
+                    }
                 });
                 pipeline_reads_and_fmas<G::plan.nsrc, plan_fma_count(G::plan, L)>();
                 if constexpr (G::CLS == CLS_H) {
