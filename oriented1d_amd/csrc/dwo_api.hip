@@ -92,6 +92,19 @@ int try_plane_wgrad(const void *x, const void *dy, const void *taps, float *part
     return -100;
 }
 
+// NHWC with the channel count a multiple of 4, stride 1, at the same extents: the slice kernels
+template <typename T>
+int try_nhwc_plane_conv(int op, const void *src, const float *w, const float *bias,
+                        const void *taps, void *dst, const ConvDims &d, int layout, hipStream_t st) {
+    if (layout != DWO_NHWC || d.stride != 1 || d.C % kSliceCh != 0) return -100;
+#define DWO_MATCH(K_, H_, W_)                                                                    \
+    if (d.K == K_ && d.H == H_ && d.W == W_)                                                     \
+        return launch_nhwc_plane_conv<T, K_, H_, W_>(op, src, w, bias, taps, dst, d.N, d.C, st);
+    DWO_PLANE_SHAPES(DWO_MATCH)
+#undef DWO_MATCH
+    return -100;
+}
+
 // NHWC with a kernel size that has lane-resident tap kernels; -100 otherwise
 #define DWO_NHWC_KS(X) X(7) X(13) X(15) X(27) X(31)
 bool nhwc_has_k(int K) {
@@ -104,7 +117,33 @@ bool nhwc_has_k(int K) {
 // wgrad partial-sum count per (channel, tap): an upper bound that sizes the scratch buffer
 // (the staged path picks its group count from the device's occupancy at launch, never more
 // than kMaxPlaneGroups nor than the number of staged batches).
+// images per staged batch of the NHWC slice kernels, 0 when they do not cover the shape
+int nhwc_plane_batch(const ConvDims &d, int layout) {
+    if (layout != DWO_NHWC || d.stride != 1 || d.C % kSliceCh != 0) return 0;
+#define DWO_MATCH(K_, H_, W_) \
+    if (d.K == K_ && d.H == H_ && d.W == W_) return NhwcTile<H_, W_>::PBI;
+    DWO_PLANE_SHAPES(DWO_MATCH)
+#undef DWO_MATCH
+    return 0;
+}
+
+template <typename T>
+int try_nhwc_plane_wgrad(const void *x, const void *dy, const void *taps, float *part, int *groups,
+                         const ConvDims &d, hipStream_t st) {
+#define DWO_MATCH(K_, H_, W_)                                                                    \
+    if (d.K == K_ && d.H == H_ && d.W == W_)                                                     \
+        return launch_nhwc_plane_wgrad<T, K_, H_, W_>(x, dy, taps, part, d.N, d.C, groups, st);
+    DWO_PLANE_SHAPES(DWO_MATCH)
+#undef DWO_MATCH
+    return -100;
+}
+
 int wgrad_max_partials(const ConvDims &d, int layout) {
+    const int PBI = nhwc_plane_batch(d, layout);
+    if (PBI != 0) {
+        const int nbatch = (d.N + PBI - 1) / PBI;
+        return nbatch < kMaxPlaneGroups ? nbatch : kMaxPlaneGroups;
+    }
     const int PB = plane_batch(d, layout);
     if (PB == 0 && layout == DWO_NHWC && nhwc_has_k(d.K)) {
         int ppw = 0;
@@ -155,6 +194,8 @@ int fprop_t(const void *x, const float *w, const float *bias, const void *taps, 
             const ConvDims &d, int layout, hipStream_t st) {
     const int fast = try_plane_conv<T>(OP_FPROP, x, w, bias, taps, y, d, layout, st);
     if (fast != -100) return fast;
+    const int sliced = try_nhwc_plane_conv<T>(OP_FPROP, x, w, bias, taps, y, d, layout, st);
+    if (sliced != -100) return sliced;
     const int nhwc = try_nhwc_conv<T, NHWC_FPROP>(x, w, bias, taps, y, d, layout, st);
     if (nhwc != -100) return nhwc;
     const int total = d.N * d.C * d.P * d.Q;
@@ -174,6 +215,8 @@ int dgrad_t(const void *dy, const float *w, const void *taps, void *dx, const Co
             int layout, hipStream_t st) {
     const int fast = try_plane_conv<T>(OP_DGRAD, dy, w, nullptr, taps, dx, d, layout, st);
     if (fast != -100) return fast;
+    const int sliced = try_nhwc_plane_conv<T>(OP_DGRAD, dy, w, nullptr, taps, dx, d, layout, st);
+    if (sliced != -100) return sliced;
     const int nhwc = try_nhwc_conv<T, NHWC_DGRAD>(dy, w, nullptr, taps, dx, d, layout, st);
     if (nhwc != -100) return nhwc;
     const int total = d.N * d.C * d.H * d.W;
@@ -195,6 +238,8 @@ int wgrad_t(const void *dy, const void *x, const void *taps, float *dw, float *d
     int rc, NG = 0;
     if (plane_batch(d, layout) != 0) {
         rc = try_plane_wgrad<T>(x, dy, taps, part, &NG, d, st);
+    } else if (nhwc_plane_batch(d, layout) != 0) {
+        rc = try_nhwc_plane_wgrad<T>(x, dy, taps, part, &NG, d, st);
     } else if (layout == DWO_NHWC && nhwc_has_k(d.K)) {
         rc = try_nhwc_wgrad<T>(dy, x, taps, part, &NG, d, st);
     } else {

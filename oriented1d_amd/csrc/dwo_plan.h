@@ -179,6 +179,7 @@ constexpr int pair_plan_dot_count(const PairPlan &p, int L) {
 
 constexpr int round_up(int v, int m) { return (v + m - 1) / m * m; }
 constexpr int cmax(int a, int b) { return a > b ? a : b; }
+constexpr int cmin(int a, int b) { return a < b ? a : b; }
 
 // Smallest r >= need with (mult * r - target) divisible by 32, or need rounded to odd when
 // no such r exists within one period.  Used to pick LDS row strides for which the flattened
@@ -284,5 +285,30 @@ constexpr int tile_L(int o) {
     return orient_class(o) == CLS_H ? Tile<H, W>::LH
                                     : (orient_class(o) == CLS_V ? Tile<H, W>::LV : Tile<H, W>::LD);
 }
+
+// NHWC slice kernels: a workgroup owns kSliceCh consecutive channels.
+constexpr int kSliceCh = 4;
+// Threads per workgroup and images staged per batch: sized so that a sub-group (NT / kSliceCh
+// threads) sees 2 to 4 items per thread and the planes of a batch fit in LDS.
+template <int H, int W>
+struct NhwcTile {
+    static constexpr int NT = 256, PBI = 1;
+};
+template <>
+struct NhwcTile<56, 56> {
+    static constexpr int NT = 1024, PBI = 1;
+};
+template <>
+struct NhwcTile<28, 28> {
+    static constexpr int NT = 512, PBI = 1;
+};
+template <>
+struct NhwcTile<14, 14> {
+    static constexpr int NT = 512, PBI = 2;
+};
+template <>
+struct NhwcTile<7, 7> {
+    static constexpr int NT = 512, PBI = 4;
+};
 
 }  // namespace dwo

@@ -49,6 +49,9 @@ struct Vec4<float> {
     __device__ __forceinline__ void store(float *p) const {
         __builtin_nontemporal_store(v, reinterpret_cast<f4 *>(p));
     }
+    // through the caches: for lines that other workgroups touch at about the same time
+    __device__ __forceinline__ void load_cached(const float *p) { v = *reinterpret_cast<const f4 *>(p); }
+    __device__ __forceinline__ void store_cached(float *p) const { *reinterpret_cast<f4 *>(p) = v; }
     __device__ __forceinline__ float get(int i) const { return v[i]; }
     __device__ __forceinline__ uint16_t bits(int) const { return 0; }
     __device__ __forceinline__ void set(float a, float b, float c, float d) {
@@ -65,6 +68,8 @@ struct Vec4<bf16_t> {
     __device__ __forceinline__ void store(bf16_t *p) const {
         __builtin_nontemporal_store(v, reinterpret_cast<u2 *>(p));
     }
+    __device__ __forceinline__ void load_cached(const bf16_t *p) { v = *reinterpret_cast<const u2 *>(p); }
+    __device__ __forceinline__ void store_cached(bf16_t *p) const { *reinterpret_cast<u2 *>(p) = v; }
     __device__ __forceinline__ float get(int i) const {
         const uint32_t w = i < 2 ? v.x : v.y;
         return __uint_as_float((i & 1) ? (w & 0xffff0000u) : (w << 16));
@@ -87,6 +92,8 @@ struct Vec4<f16_t> {
     __device__ __forceinline__ void store(f16_t *p) const {
         __builtin_nontemporal_store(v, reinterpret_cast<h4 *>(p));
     }
+    __device__ __forceinline__ void load_cached(const f16_t *p) { v = *reinterpret_cast<const h4 *>(p); }
+    __device__ __forceinline__ void store_cached(f16_t *p) const { *reinterpret_cast<h4 *>(p) = v; }
     __device__ __forceinline__ float get(int i) const { return (float)v[i]; }
     __device__ __forceinline__ uint16_t bits(int i) const {
         return __builtin_bit_cast(uint16_t, (_Float16)v[i]);
@@ -345,6 +352,72 @@ struct ConvStagers {
     }
 };
 
+// Weights of one channel for a canonical geometry G, duplicates folded into their
+// representative tap (and packed two taps to a word when PAIR), plus the bias; accumulate()
+// is the straight-line body of one item: G::plan.nsrc LDS reads feeding L accumulators.
+template <class G, int OP, typename T, int K, bool PAIR>
+struct ChannelTaps {
+    static constexpr int L = G::L_;
+    static constexpr int NPAIR = [] {
+        if constexpr (PAIR) return cmax((int)G::plan.npair, 1);
+        else return 1;
+    }();
+    float wv[K];
+    unsigned wp[NPAIR];
+    float bv;
+
+    __device__ __forceinline__ void load(const float *__restrict__ wt, const float *__restrict__ bias,
+                                         int c) {
+        const float *wc = wt + (size_t)c * K;
+#pragma unroll
+        for (int s = 0; s < K; s++) wv[s] = wc[OP == OP_DGRAD ? K - 1 - s : s];
+        static_for<K>([&](auto s) {
+            constexpr int r = G::plan.rep[s];
+            if constexpr (r >= 0 && r != s) wv[r] += wv[s];
+        });
+        // folded sums are uniform: move them back to scalar registers
+        static_for<K>([&](auto s) {
+            if constexpr (s > 0 && G::plan.rep[s] >= 0 && G::plan.rep[s] != s) {
+                constexpr int r = G::plan.rep[s];
+                wv[r] = __builtin_bit_cast(
+                    float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, wv[r])));
+            }
+        });
+        bv = (OP == OP_FPROP && bias != nullptr) ? bias[c] : 0.f;
+        // pair form: (tap, next tap along the run) as two 16-bit weights per uniform word
+        if constexpr (PAIR) {
+            static_for<NPAIR>([&](auto q) {
+                constexpr int lo = G::plan.pair_lo[q], hi = G::plan.pair_hi[q];
+                unsigned v = raw16(from_float<T>(wv[lo]));
+                if constexpr (hi >= 0) v |= (unsigned)raw16(from_float<T>(wv[hi])) << 16;
+                wp[q] = __builtin_amdgcn_readfirstlane(v);
+            });
+        }
+    }
+
+    __device__ __forceinline__ void accumulate(const float *base, float (&acc)[L]) const {
+#pragma unroll
+        for (int l = 0; l < L; l++) acc[l] = bv;
+        static_for<G::plan.nsrc>([&](auto m) {
+            constexpr int off = G::imm(G::plan.sh[m], G::plan.sw[m]);
+            if constexpr (PAIR) {
+                const unsigned v = reinterpret_cast<const unsigned *>(base)[off];
+                static_for<L>([&](auto l) {
+                    constexpr int q = G::plan.user[m][l];
+                    if constexpr (q >= 0) acc[l] = dot2_acc(v, wp[q], acc[l], T{});
+                });
+            } else {
+                const float v = base[off];
+                static_for<L>([&](auto l) {
+                    constexpr int t = G::plan.user[m][l];
+                    if constexpr (t >= 0) acc[l] = __builtin_fmaf(v, wv[t], acc[l]);
+                });
+            }
+        });
+        pipeline_reads_and_fmas<G::plan.nsrc, plan_fma_count(G::plan, L)>();
+    }
+};
+
 // ---------------------------------------------------------------------------------------------
 // canonical body
 // ---------------------------------------------------------------------------------------------
@@ -375,38 +448,8 @@ __device__ __forceinline__ void run_canonical(const T *__restrict__ src, const f
     const unsigned tid = threadIdx.x;
     const unsigned pstride = (unsigned)C * (H * W);  // elements between images of one channel
 
-    // weights of this channel, duplicates folded into their representative tap
-    float wv[K];
-    const float *wc = wt + (size_t)c * K;
-#pragma unroll
-    for (int s = 0; s < K; s++) wv[s] = wc[OP == OP_DGRAD ? K - 1 - s : s];
-    static_for<K>([&](auto s) {
-        constexpr int r = G::plan.rep[s];
-        if constexpr (r >= 0 && r != s) wv[r] += wv[s];
-    });
-    // folded sums are uniform: move them back to scalar registers
-    static_for<K>([&](auto s) {
-        if constexpr (s > 0 && G::plan.rep[s] >= 0 && G::plan.rep[s] != s) {
-            constexpr int r = G::plan.rep[s];
-            wv[r] = __builtin_bit_cast(
-                float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, wv[r])));
-        }
-    });
-    const float bv = (OP == OP_FPROP && bias != nullptr) ? bias[c] : 0.f;
-    // pair form: (tap, next tap along the run) as two 16-bit weights per uniform word
-    constexpr int NPAIR = [] {
-        if constexpr (PAIR) return cmax((int)G::plan.npair, 1);
-        else return 1;
-    }();
-    unsigned wp[NPAIR];
-    if constexpr (PAIR) {
-        static_for<NPAIR>([&](auto q) {
-            constexpr int lo = G::plan.pair_lo[q], hi = G::plan.pair_hi[q];
-            unsigned v = raw16(from_float<T>(wv[lo]));
-            if constexpr (hi >= 0) v |= (unsigned)raw16(from_float<T>(wv[hi])) << 16;
-            wp[q] = __builtin_amdgcn_readfirstlane(v);
-        });
-    }
+    ChannelTaps<G, OP, T, K, PAIR> taps;
+    taps.load(wt, bias, c);
 
     // zero the staging area once; interiors are overwritten per batch, halos stay zero
     for (unsigned i = tid; i < PB * PLS; i += NT) lds[i] = 0.f;
@@ -441,25 +484,7 @@ __device__ __forceinline__ void run_canonical(const T *__restrict__ src, const f
             if (item < PB * G::IPP && (int)pl < nvalid) {
                 const float *base = lds + (pl * PLS + rb * (G::LR * G::RS) + j);
                 float acc[L];
-#pragma unroll
-                for (int l = 0; l < L; l++) acc[l] = bv;
-                static_for<G::plan.nsrc>([&](auto m) {
-                    constexpr int off = G::imm(G::plan.sh[m], G::plan.sw[m]);
-                    if constexpr (PAIR) {
-                        const unsigned v = reinterpret_cast<const unsigned *>(base)[off];
-                        static_for<L>([&](auto l) {
-                            constexpr int q = G::plan.user[m][l];
-                            if constexpr (q >= 0) acc[l] = dot2_acc(v, wp[q], acc[l], T{});
-                        });
-                    } else {
-                        const float v = base[off];
-                        static_for<L>([&](auto l) {
-                            constexpr int t = G::plan.user[m][l];
-                            if constexpr (t >= 0) acc[l] = __builtin_fmaf(v, wv[t], acc[l]);
-                        });
-                    }
-                });
-                pipeline_reads_and_fmas<G::plan.nsrc, plan_fma_count(G::plan, L)>();
+                taps.accumulate(base, acc);
                 if constexpr (G::CLS == CLS_H) {
                     T *o = obase + (pl * pstride + rb * W + j * L);
                     if constexpr (L == 4) {
