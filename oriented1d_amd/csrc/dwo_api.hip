@@ -8,6 +8,7 @@
 #include "dwo_generic.h"
 #include "dwo_nhwc.h"
 #include "dwo_dispatch.h"
+#include "dwo_nhwc_tile.h"
 
 using namespace dwo;
 
@@ -154,6 +155,15 @@ int wgrad_max_partials(const ConvDims &d, int layout) {
     return nbatch < kMaxPlaneGroups ? nbatch : kMaxPlaneGroups;
 }
 
+// NHWC fprop at any extent and stride with the channel count a multiple of 4: slice tiles
+template <typename T>
+int try_nhwc_tile_fprop(const void *x, const float *w, const float *bias, const void *taps, void *y,
+                        const ConvDims &d, int layout, hipStream_t st) {
+    if (layout != DWO_NHWC || d.C % kSliceCh != 0) return -100;
+    if ((size_t)d.H * d.W * d.C * sizeof(T) >= 0xffffffffull) return -100;  // 32-bit image offsets
+    return launch_nhwc_tile_fprop<T>(x, w, bias, taps, y, d, st);
+}
+
 template <typename T, int MODE>
 int try_nhwc_conv(const void *src, const float *w, const float *bias, const void *taps, void *dst,
                   const ConvDims &d, int layout, hipStream_t st) {
@@ -196,6 +206,8 @@ int fprop_t(const void *x, const float *w, const float *bias, const void *taps, 
     if (fast != -100) return fast;
     const int sliced = try_nhwc_plane_conv<T>(OP_FPROP, x, w, bias, taps, y, d, layout, st);
     if (sliced != -100) return sliced;
+    const int tiled = try_nhwc_tile_fprop<T>(x, w, bias, taps, y, d, layout, st);
+    if (tiled != -100) return tiled;
     const int nhwc = try_nhwc_conv<T, NHWC_FPROP>(x, w, bias, taps, y, d, layout, st);
     if (nhwc != -100) return nhwc;
     const int total = d.N * d.C * d.P * d.Q;

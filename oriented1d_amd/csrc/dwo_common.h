@@ -77,6 +77,13 @@ __device__ __forceinline__ float wave_sum(float v) {
     return v;
 }
 
+// Dynamic LDS beyond 64 KB has to be allowed per kernel before the first launch.
+template <class Kern>
+void allow_large_lds(Kern kern, size_t lds) {
+    (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+}
+
 struct ConvDims {
     int N, C, H, W, P, Q, K, stride, shift;  // shift = log2(stride)
 };

@@ -298,12 +298,6 @@ __global__ __launch_bounds__((NhwcTile<H, W>::NT)) void nhwc_plane_kernel(
 #undef DWO_CASE
 }
 
-template <class Kern>
-void allow_large_lds(Kern kern, size_t lds) {
-    (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-}
-
 // C must be a multiple of kSliceCh (the caller checks).
 template <typename T, int K, int H, int W>
 int launch_nhwc_plane_conv(int op, const void *src, const float *w, const float *bias,

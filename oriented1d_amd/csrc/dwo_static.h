@@ -53,6 +53,8 @@ struct Vec4<float> {
     __device__ __forceinline__ void load_cached(const float *p) { v = *reinterpret_cast<const f4 *>(p); }
     __device__ __forceinline__ void store_cached(float *p) const { *reinterpret_cast<f4 *>(p) = v; }
     __device__ __forceinline__ float get(int i) const { return v[i]; }
+    __device__ __forceinline__ float elem(int i) const { return v[i]; }
+    __device__ __forceinline__ void clear() { v = f4{0.f, 0.f, 0.f, 0.f}; }
     __device__ __forceinline__ uint16_t bits(int) const { return 0; }
     __device__ __forceinline__ void set(float a, float b, float c, float d) {
         v[0] = a, v[1] = b, v[2] = c, v[3] = d;
@@ -77,6 +79,8 @@ struct Vec4<bf16_t> {
     __device__ __forceinline__ uint16_t bits(int i) const {
         return (uint16_t)((i < 2 ? v.x : v.y) >> (16 * (i & 1)));
     }
+    __device__ __forceinline__ bf16_t elem(int i) const { return bf16_t{bits(i)}; }
+    __device__ __forceinline__ void clear() { v = u2{0u, 0u}; }
     __device__ __forceinline__ void set(float a, float b, float c, float d) {
         v.x = (uint32_t)from_float<bf16_t>(a).bits | ((uint32_t)from_float<bf16_t>(b).bits << 16);
         v.y = (uint32_t)from_float<bf16_t>(c).bits | ((uint32_t)from_float<bf16_t>(d).bits << 16);
@@ -95,6 +99,8 @@ struct Vec4<f16_t> {
     __device__ __forceinline__ void load_cached(const f16_t *p) { v = *reinterpret_cast<const h4 *>(p); }
     __device__ __forceinline__ void store_cached(f16_t *p) const { *reinterpret_cast<h4 *>(p) = v; }
     __device__ __forceinline__ float get(int i) const { return (float)v[i]; }
+    __device__ __forceinline__ f16_t elem(int i) const { return v[i]; }
+    __device__ __forceinline__ void clear() { v = h4{0, 0, 0, 0}; }
     __device__ __forceinline__ uint16_t bits(int i) const {
         return __builtin_bit_cast(uint16_t, (_Float16)v[i]);
     }

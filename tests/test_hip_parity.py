@@ -116,6 +116,17 @@ def test_strided_and_odd_extents(oracle, stride, H, W, K, nhwc, dtype):
     _case(oracle, 2, 64, H, W, K, stride, dtype, nhwc, grouped_theta(64), seed=H * W + K)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("stride,H,W,K", [(2, 150, 138, 31), (1, 70, 200, 15), (4, 97, 64, 27)])
+def test_nhwc_large_planes_many_tiles(oracle, stride, H, W, K, dtype):
+    """NHWC planes that take several bands and sub-tiles per workgroup; the eight canonical
+    orientations in channel groups of four plus one group of arbitrary angles (mixed tap extents
+    inside a slice)."""
+    theta = np.concatenate([np.repeat(canonical_theta(8), 4),
+                            np.array([0.3, 1.1, 2.0, 2.9], dtype=np.float32)]).astype(np.float32)
+    _case(oracle, 2, 36, H, W, K, stride, dtype, True, theta, seed=H + W + K)
+
+
 @pytest.mark.parametrize("nhwc", [False, True], ids=["nchw", "nhwc"])
 def test_random_angles_ragged_shapes(oracle, nhwc):
     rng = np.random.default_rng(77)
