@@ -31,7 +31,8 @@ def hipcc():
     return exe
 
 
-PLANE_SHAPES = [(31, 56, 56), (31, 28, 28), (31, 14, 14), (31, 7, 7)]  # = DWO_PLANE_SHAPES
+PLANE_SHAPES = [(31, 56, 56), (31, 28, 28), (31, 14, 14), (31, 7, 7),
+                (15, 56, 56), (15, 28, 28), (15, 14, 14), (15, 7, 7)]  # = DWO_PLANE_SHAPES
 PLANE_TYPES = ["float", "bf16_t", "f16_t"]
 
 

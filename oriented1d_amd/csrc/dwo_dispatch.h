@@ -8,9 +8,13 @@
 #include "dwo_common.h"
 #include "dwo_plan.h"
 
-// X(K, H, W): kernel size and plane extents with compile-time kernels (NCHW, stride 1)
+// X(K, H, W): kernel size and plane extents with compile-time kernels (stride 1): the ConvNeXt
+// stage extents at 224 x 224 input for K = 31 (1D blocks, second conv of 1D++ blocks) and K = 15
+// (first conv of 1D++ blocks)
 #ifndef DWO_PLANE_SHAPES
-#define DWO_PLANE_SHAPES(X) X(31, 56, 56) X(31, 28, 28) X(31, 14, 14) X(31, 7, 7)
+#define DWO_PLANE_SHAPES(X)                                   \
+    X(31, 56, 56) X(31, 28, 28) X(31, 14, 14) X(31, 7, 7)     \
+    X(15, 56, 56) X(15, 28, 28) X(15, 14, 14) X(15, 7, 7)
 #endif
 
 namespace dwo {

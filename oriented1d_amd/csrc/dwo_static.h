@@ -120,7 +120,8 @@ constexpr int max_plane_floats(std::integer_sequence<int, Os...>) {
     constexpr int PAD = table_pad<K, H, W>();
     int m = (H + 2 * PAD) * (W + 2 * PAD + 3);  // table-driven body
     ((m = cmax(m, Geo<Os, K, tile_L<H, W>(Os), H, W>::PLANE)), ...);
-    ((m = cmax(m, Geo<Os, K, tile_L<H, W>(Os), H, W, true>::PLANE)), ...);
+    // (pair geometries exist for row-direction orientations only, see use_pairs)
+    ((m = cmax(m, orient_class(Os) == CLS_H ? Geo<Os, K, tile_L<H, W>(Os), H, W, true>::PLANE : 0)), ...);
     return m;
 }
 template <int K, int H, int W>

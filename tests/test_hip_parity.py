@@ -88,6 +88,15 @@ def test_stage_shapes_k31(oracle, C, HW, nhwc, dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("nhwc", [False, True], ids=["nchw", "nhwc"])
+@pytest.mark.parametrize("C,HW", [(64, 56), (128, 28), (256, 14), (512, 7)])
+def test_stage_shapes_k15(oracle, C, HW, nhwc, dtype):
+    """First convolution of the 1D++ blocks: K = 15 at the stage extents, contiguous-group
+    angles with the +90 degree offset of odd layers."""
+    _case(oracle, 3, C, HW, HW, 15, 1, dtype, nhwc, grouped_theta(C, 0.5), seed=C + HW + 15)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
 @pytest.mark.parametrize("C,HW", [(40, 56), (40, 28), (72, 14), (100, 7)])
 def test_stage_shapes_mixed_angles(oracle, C, HW, dtype):
     """Stage plane extents with arbitrary angles mixed among canonical ones (a workgroup picks
