@@ -52,6 +52,8 @@ def main():
     ap.add_argument("--kernel-repeats", type=int, default=7,
                     help="repeats of the per-kernel measurement (the median is reported)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-extra-sweeps", action="store_true",
+                    help="skip the bf16 / NHWC / grouped-angle rows (other_configs)")
     ap.add_argument("--only", default="", help="restrict the per-kernel table, e.g. 96x56:fprop")
     ap.add_argument("--model-iters", type=int, default=5,
                     help="timed ConvNeXt-T-1D inference forwards (batch 128, bf16); 0 skips it")
@@ -73,125 +75,129 @@ def main():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(2)
     dev = torch.device("cuda:0")
-    tdt = {"f32": torch.float32, "bf16": torch.bfloat16, "f16": torch.float16}[args.dtype]
-    b = ELEM[args.dtype]
-    nhwc = args.layout == "nhwc"
 
-    def theta_for(C):
-        if args.theta == "roundrobin":
-            return np.array([(c % 8) * math.pi / 8 for c in range(C)], dtype=np.float32)
-        return np.array([math.pi * (((8 * (c + 1) - 1) // C) / 8) for c in range(C)],
-                        dtype=np.float32)
-
-    # ------------------------------------------------------------------ resident inputs
-    g = torch.Generator(device=dev).manual_seed(0)
-    bytes_per_set = sum(3 * BATCH * C * HW * HW * b for C, HW in STAGES)
-    nsets = max(2, math.ceil(2 * 256e6 / (2 * BATCH * 96 * 56 * 56 * b)) + 1)
-    sets = []
-    for _ in range(nsets):
-        st = []
-        for C, HW in STAGES:
-            shape = (BATCH, HW, HW, C) if nhwc else (BATCH, C, HW, HW)
-            x = torch.randn(shape, device=dev, generator=g).to(tdt)
-            dy = torch.randn(shape, device=dev, generator=g).to(tdt)
-            w = torch.randn(C, 1, 1, KSIZE, device=dev, generator=g) * 0.02
-            taps = op.build_taps(torch.from_numpy(theta_for(C)), C, KSIZE).to(dev)
-            st.append((C, HW, x, dy, w, taps))
-        sets.append(st)
-
-    # Outputs and wgrad scratch are allocated once; the timed region holds nothing but the
-    # C-ABI calls (ctypes arguments are converted up front).
     import ctypes
 
     from oriented1d_amd import _lib
     lib = _lib.load()
-    stream_h = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
-    dt_code, lay_code = {"f32": 0, "bf16": 1, "f16": 2}[args.dtype], int(nhwc)
-    keep = []
+    stream = torch.cuda.current_stream(dev)
+    stream_h = ctypes.c_void_p(stream.cuda_stream)
+
+    def theta_for(C, kind):
+        if kind == "roundrobin":
+            return np.array([(c % 8) * math.pi / 8 for c in range(C)], dtype=np.float32)
+        return np.array([math.pi * (((8 * (c + 1) - 1) // C) / 8) for c in range(C)],
+                        dtype=np.float32)
 
     def vp(t):
         return ctypes.c_void_p(t.data_ptr())
 
-    calls = []  # calls[set][stage][op] -> zero-argument callable
-    for st in sets:
-        per_stage = []
-        for (C, HW, x, dy, w, taps) in st:
-            w2 = w.reshape(C, KSIZE).contiguous()
-            y = torch.empty_like(x)
-            dx = torch.empty_like(x)
-            dw = torch.empty(C, KSIZE, device=dev)
-            nb = lib.dwo_wgrad_scratch_bytes(BATCH, C, HW, HW, KSIZE, 1, dt_code, lay_code)
-            scr = torch.empty(max(nb, 16), dtype=torch.uint8, device=dev)
-            keep.extend([w2, y, dx, dw, scr])
-            dims = (BATCH, C, HW, HW, KSIZE, 1, dt_code, lay_code, stream_h)
-            fa = (vp(x), vp(w2), None, vp(taps), vp(y)) + dims
-            da = (vp(dy), vp(w2), vp(taps), vp(dx)) + dims
-            wa = (vp(dy), vp(x), vp(taps), vp(dw), None, vp(scr), nb) + dims
-            per_stage.append({
-                "fprop": (lambda a=fa: lib.dwo_fprop(*a)),
-                "dgrad": (lambda a=da: lib.dwo_dgrad(*a)),
-                "wgrad": (lambda a=wa: lib.dwo_wgrad(*a)),
-            })
-        calls.append(per_stage)
-    for per_stage in calls:  # one checked pass: any launch error surfaces here
-        for ops in per_stage:
+    def sweep(dtype, layout, theta, steps, warmup, kernel_iters, kernel_repeats, only="",
+              warm=False):
+        """Whole-step time (when steps > 0) and per-(shape, op) kernel times of one
+        configuration.  Inputs are resident before anything is timed; nsets buffer sets rotate
+        so consecutive launches do not re-hit the 256 MB Infinity Cache ("cold" numbers); with
+        warm=True every launch of an operator also runs on one fixed set ("warm_us")."""
+        tdt = {"f32": torch.float32, "bf16": torch.bfloat16, "f16": torch.float16}[dtype]
+        b = ELEM[dtype]
+        nhwc = layout == "nhwc"
+        g = torch.Generator(device=dev).manual_seed(0)
+        nsets = max(2, math.ceil(2 * 256e6 / (2 * BATCH * 96 * 56 * 56 * b)) + 1)
+        dt_code, lay_code = {"f32": 0, "bf16": 1, "f16": 2}[dtype], int(nhwc)
+        keep, calls = [], []  # calls[set][stage][op] -> zero-argument callable
+        for _ in range(nsets):
+            per_stage = []
+            for C, HW in STAGES:
+                shape = (BATCH, HW, HW, C) if nhwc else (BATCH, C, HW, HW)
+                x = torch.randn(shape, device=dev, generator=g).to(tdt)
+                dy = torch.randn(shape, device=dev, generator=g).to(tdt)
+                w2 = (torch.randn(C, KSIZE, device=dev, generator=g) * 0.02).contiguous()
+                taps = op.build_taps(torch.from_numpy(theta_for(C, theta)), C, KSIZE).to(dev)
+                # outputs and wgrad scratch are allocated once; the timed region holds nothing
+                # but the C-ABI calls (ctypes arguments are converted up front)
+                y = torch.empty_like(x)
+                dx = torch.empty_like(x)
+                dw = torch.empty(C, KSIZE, device=dev)
+                nb = lib.dwo_wgrad_scratch_bytes(BATCH, C, HW, HW, KSIZE, 1, dt_code, lay_code)
+                scr = torch.empty(max(nb, 16), dtype=torch.uint8, device=dev)
+                keep.extend([x, dy, w2, taps, y, dx, dw, scr])
+                dims = (BATCH, C, HW, HW, KSIZE, 1, dt_code, lay_code, stream_h)
+                fa = (vp(x), vp(w2), None, vp(taps), vp(y)) + dims
+                da = (vp(dy), vp(w2), vp(taps), vp(dx)) + dims
+                wa = (vp(dy), vp(x), vp(taps), vp(dw), None, vp(scr), nb) + dims
+                per_stage.append({
+                    "fprop": (lambda a=fa: lib.dwo_fprop(*a)),
+                    "dgrad": (lambda a=da: lib.dwo_dgrad(*a)),
+                    "wgrad": (lambda a=wa: lib.dwo_wgrad(*a)),
+                })
+            calls.append(per_stage)
+        for ops in calls[0]:  # one checked pass: any launch error surfaces here
             for name, fn in ops.items():
                 _lib.check(fn(), "dwo_" + name)
-    torch.cuda.synchronize()
+        torch.cuda.synchronize()
 
-    def run_op(name, si, i):
-        calls[i % nsets][si][name]()
+        def step(i):
+            for ops in calls[i % nsets]:
+                ops["fprop"]()
+                ops["dgrad"]()
+                ops["wgrad"]()
 
-    def step(i):
-        for ops in calls[i % nsets]:
-            ops["fprop"]()
-            ops["dgrad"]()
-            ops["wgrad"]()
+        step_bytes = sum(algorithmic_bytes(o, BATCH, C, HW, HW, KSIZE, b)
+                         for C, HW in STAGES for o in ("fprop", "dgrad", "wgrad"))
+        ms_per_step = None
+        if steps > 0:
+            for i in range(warmup):
+                step(i)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for i in range(steps):
+                step(i)
+            torch.cuda.synchronize()
+            ms_per_step = (time.perf_counter() - t0) * 1e3 / steps
 
-    step_bytes = sum(algorithmic_bytes(o, BATCH, C, HW, HW, KSIZE, b)
-                     for C, HW in STAGES for o in ("fprop", "dgrad", "wgrad"))
-
-    # ------------------------------------------------------------------ timed steps
-    for i in range(args.warmup):
-        step(i)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for i in range(args.steps):
-        step(i)
-    torch.cuda.synchronize()
-    t1 = time.perf_counter()
-    ms_per_step = (t1 - t0) * 1e3 / args.steps
-    value = step_bytes / (ms_per_step * 1e-3) / 1e9
-
-    # ------------------------------------------------------------------ per-kernel timings
-    # HIP events on the launch stream (torch's current stream is the one passed to the C ABI).
-    detail = {}
-    stream = torch.cuda.current_stream(dev)
-    for si, (C, HW) in enumerate(STAGES):
-        for name in ("fprop", "dgrad", "wgrad"):
-            key = "%dx%d:%s" % (C, HW, name)
-            if args.only and args.only != key:
-                continue
+        # per-kernel timings: HIP events on the launch stream (torch's current stream is the
+        # one passed to the C ABI), median over the repeats
+        def timed(name, si, fixed):
             for i in range(3):
-                run_op(name, si, i)
+                calls[0 if fixed else i % nsets][si][name]()
             torch.cuda.synchronize()
             reps = []
-            for _ in range(args.kernel_repeats):
+            for _ in range(kernel_repeats):
                 e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
                 e0.record(stream)
-                for i in range(args.kernel_iters):
-                    run_op(name, si, i)
+                for i in range(kernel_iters):
+                    calls[0 if fixed else i % nsets][si][name]()
                 e1.record(stream)
                 torch.cuda.synchronize()
-                reps.append(e0.elapsed_time(e1) * 1e3 / args.kernel_iters)
-            us = sorted(reps)[len(reps) // 2]  # median of the repeats
-            ab = algorithmic_bytes(name, BATCH, C, HW, HW, KSIZE, b)
-            gbs = ab / (us * 1e-6) / 1e9
-            detail[key] = {"us": round(us, 2), "GB/s": round(gbs, 1),
-                           "frac_hbm": round(gbs / HBM_PEAK_GBS, 4), "bytes": ab}
+                reps.append(e0.elapsed_time(e1) * 1e3 / kernel_iters)
+            return sorted(reps)[len(reps) // 2]
+
+        detail = {}
+        for si, (C, HW) in enumerate(STAGES):
+            for name in ("fprop", "dgrad", "wgrad"):
+                key = "%dx%d:%s" % (C, HW, name)
+                if only and only != key:
+                    continue
+                us = timed(name, si, False)
+                ab = algorithmic_bytes(name, BATCH, C, HW, HW, KSIZE, b)
+                gbs = ab / (us * 1e-6) / 1e9
+                detail[key] = {"us": round(us, 2), "GB/s": round(gbs, 1),
+                               "frac_hbm": round(gbs / HBM_PEAK_GBS, 4), "bytes": ab}
+                if warm:
+                    detail[key]["warm_us"] = round(timed(name, si, True), 2)
+        copy_src = keep[0]
+        res = {"ms_per_step": ms_per_step, "detail": detail, "nsets": nsets,
+               "step_bytes": step_bytes, "copy_src": copy_src if args.calibration_copy else None}
+        return res
+
+    main_res = sweep(args.dtype, args.layout, args.theta, args.steps, args.warmup,
+                     args.kernel_iters, args.kernel_repeats, args.only, warm=True)
+    ms_per_step, detail = main_res["ms_per_step"], main_res["detail"]
+    nsets, step_bytes = main_res["nsets"], main_res["step_bytes"]
+    value = step_bytes / (ms_per_step * 1e-3) / 1e9
 
     if args.calibration_copy:
-        src = sets[0][0][2]
+        src = main_res["copy_src"]
         dstc = torch.empty_like(src)
         for _ in range(3):
             dstc.copy_(src)
@@ -212,8 +218,26 @@ def main():
                     "traffic": measured_traffic.get((args.dtype, args.layout, args.theta)),
                     "launch_us": dom["us"], "algorithmic_bytes": dom["bytes"]}
 
+    # ------------------------------------------------------------------ the other rows
+    # Same sweep in the other element type / layout / angle assignment (per-kernel times only,
+    # fewer repeats): bf16 NCHW, fp32 and bf16 NHWC-native, and fp32 NCHW with the networks'
+    # contiguous-group angles.
+    others = {}
+    if not args.no_extra_sweeps and not args.only:
+        for dt_, lay_, th_ in (("bf16", "nchw", "roundrobin"), ("f32", "nhwc", "roundrobin"),
+                               ("bf16", "nhwc", "roundrobin"), ("f32", "nchw", "grouped")):
+            if (dt_, lay_, th_) == (args.dtype, args.layout, args.theta):
+                continue
+            r = sweep(dt_, lay_, th_, 0, 0, max(5, args.kernel_iters // 2), 3)
+            tot_us = sum(v["us"] for v in r["detail"].values())
+            others["%s/%s/%s" % (dt_, lay_, th_)] = {
+                "sum_us": round(tot_us, 1),
+                "GB/s": round(r["step_bytes"] / tot_us / 1e3, 1),
+                "ops": {k: [v["us"], v["frac_hbm"]] for k, v in r["detail"].items()}}
+            torch.cuda.empty_cache()
+
     # ------------------------------------------------------------------ CPU baseline (oracle)
-    cpu = None
+    cpu, cpu_all = None, None
     if not args.no_cpu_baseline:
         from oracle import dwo_oracle as oracle
 
@@ -221,7 +245,7 @@ def main():
         n_cpu = BATCH  # the whole step once: every stage shape at batch 64, all three ops
         cpu_bytes, cpu_s = 0, 0.0
         for C, HW in STAGES:
-            th = theta_for(C)
+            th = theta_for(C, args.theta)
             x = rng.standard_normal((n_cpu, C, HW, HW)).astype(np.float32)
             dy = rng.standard_normal((n_cpu, C, HW, HW)).astype(np.float32)
             w = (rng.standard_normal((C, 1, 1, KSIZE)) * 0.02).astype(np.float32)
@@ -232,6 +256,23 @@ def main():
             cpu_s += time.perf_counter() - c0
             cpu_bytes += sum(algorithmic_bytes(o, n_cpu, C, HW, HW, KSIZE, 4)
                              for o in ("fprop", "dgrad", "wgrad"))
+        # the same loops with the channels spread over all host threads (the reference has no
+        # threaded CPU path; reported for scale), on the largest stage only
+        nthr = oracle.max_threads()
+        C, HW = STAGES[0]
+        th = theta_for(C, args.theta)
+        x = rng.standard_normal((n_cpu, C, HW, HW)).astype(np.float32)
+        w = (rng.standard_normal((C, 1, 1, KSIZE)) * 0.02).astype(np.float32)
+        c0 = time.perf_counter()
+        oracle.fprop(x, w, th, acc="f32", threads=nthr)
+        oracle.dgrad(x, w, th, acc="f32", threads=nthr)
+        oracle.wgrad(x, x, th, KSIZE, acc="f32", threads=nthr)
+        mt_s = time.perf_counter() - c0
+        mt_bytes = sum(algorithmic_bytes(o, n_cpu, C, HW, HW, KSIZE, 4)
+                       for o in ("fprop", "dgrad", "wgrad"))
+        cpu_all = {"value": round(mt_bytes / mt_s / 1e9, 3), "unit": "GB/s", "cores": nthr,
+                   "sample": "fprop+dgrad+wgrad at C=96, 56x56, batch 64, channels over %d "
+                             "threads (%.1f s)" % (nthr, mt_s)}
         cpu = {"value": round(cpu_bytes / cpu_s / 1e9, 4), "unit": "GB/s", "cores": 1,
                "kind": "port",
                "sample": "one whole step: fp32 fprop+dgrad+wgrad at each of the four stage shapes, "
@@ -245,7 +286,7 @@ def main():
     # the host, fp32, batch 8, oriented convs by the oracle) is reported beside it.
     model_info = None
     if args.model_iters > 0:
-        del sets, calls, keep
+        main_res = None
         torch.cuda.empty_cache()
         from oriented1d_amd.convnext1d import convnext_tiny_1d
         from oriented1d_amd.dwoconv1d import DepthwiseOrientedConv1d
@@ -312,6 +353,7 @@ def main():
                    "algorithmic_bytes_per_step": step_bytes},
         "frac_hbm_peak": round(value / HBM_PEAK_GBS, 4),
         "detail": detail, "roofline": roofline, "cpu_baseline": cpu,
+        "cpu_baseline_all_threads": cpu_all, "other_configs": others,
         "convnext_t_1d": model_info,
     }
     print(json.dumps(out))
