@@ -62,8 +62,8 @@ def main():
                          "of known traffic, for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
-        print("bench.py: this build measures one GPU only (the operator has no cross-GPU "
-              "exchange; see DESIGN.md on sharding); run with --gpus 1", file=sys.stderr)
+        print("bench.py: this build measures one GPU only (fprop and dgrad have no cross-GPU "
+              "exchange, wgrad would need one all-reduce of dw); run with --gpus 1", file=sys.stderr)
         sys.exit(2)
 
     import numpy as np
@@ -207,7 +207,7 @@ def main():
     # scaled by what the same counter reads for a plain copy of known size (summary and the
     # commands under profiles/dwoconv1d_stage_sweep_f32_nchw_hbm_traffic.md); only valid for
     # the configuration it was measured on.
-    measured_traffic = {("f32", "nchw", "roundrobin"): int((76145 + 80576) * 1024)}
+    measured_traffic = {("f32", "nchw", "roundrobin"): 160493234}
 
     dom = detail.get("96x56:fprop")
     roofline = None
