@@ -19,6 +19,10 @@ from .dwoconv1d import DepthwiseOrientedConv1d
 
 # (block kernel sizes, stem kernel size) per variant -- models/convnext.py:485-492
 _VARIANTS = {"1d": ((31,), 31), "1dpp": ((15, 31), 15)}
+# per-stage block kernel sizes of the dense-prediction backbone (cropped for the coarse stages)
+# -- semantic_segmentation/backbone/convnext.py:316-327
+_BACKBONE_BLOCK_SIZES = {"1d": ((31,), (31,), (27,), (13,)),
+                         "1dpp": ((15, 31), (15, 31), (15, 27), (13, 13))}
 
 
 def channel_angles(channels, n_dir=8, layer_offset=0.0):
@@ -29,14 +33,28 @@ def channel_angles(channels, n_dir=8, layer_offset=0.0):
             for c in range(channels)]
 
 
+class ConvWrapper(nn.Module):
+    """Holds the operator as ``.conv``: the backbone's parameter naming
+    (semantic_segmentation/backbone/convnext.py:74-80)."""
+
+    def __init__(self, conv):
+        super().__init__()
+        self.conv = conv
+
+    def forward(self, x):
+        return self.conv(x)
+
+
 def oriented_conv(channels, kernel_size, *, stride=1, padding=None, n_dir=8, layer_offset=0.0,
-                  nhwc=False, resid=False, arbitrary_size=False):
-    """models/convnext.py:80-128 (get_convolution_1d)."""
-    return DepthwiseOrientedConv1d(
+                  nhwc=False, resid=False, arbitrary_size=False, wrapped=False):
+    """models/convnext.py:80-128 (get_convolution_1d); ``wrapped`` gives the backbone's form
+    (semantic_segmentation/backbone/convnext.py:82-104: arbitrary sizes, inside a wrapper)."""
+    conv = DepthwiseOrientedConv1d(
         channels, channels, kernel_size, groups=channels, stride=stride,
         padding=kernel_size // 2 if padding is None else padding, bias=True,
         angle=channel_angles(channels, n_dir, layer_offset), nhwc=nhwc, resid=resid,
-        arbitrary_size=arbitrary_size)
+        arbitrary_size=arbitrary_size or wrapped)
+    return ConvWrapper(conv) if wrapped else conv
 
 
 def _odd_layer_offset(index):
@@ -77,15 +95,17 @@ class Stem1D(nn.Module):
     """3 -> dim1 pointwise, two stride-2 oriented convs (NHWC) with LayerNorm + GELU, dim1 -> dim2
     pointwise, LayerNorm; NCHW in, NCHW out at 1/4 resolution (models/convnext.py:132-191)."""
 
-    def __init__(self, dim0, dim1, dim2, kernel_size, arbitrary_size=False):
+    def __init__(self, dim0, dim1, dim2, kernel_size, arbitrary_size=False, wrapped=False):
         super().__init__()
         self.pw1 = nn.Linear(dim0, dim1)
         self.pw2 = nn.Linear(dim1, dim2)
         pad = (kernel_size - 2) // 2  # shapes the parent Conv2d only; compute pads K // 2
         self.dw1 = oriented_conv(dim1, kernel_size, stride=2, padding=pad, nhwc=True,
-                                 layer_offset=_odd_layer_offset(0), arbitrary_size=arbitrary_size)
+                                 layer_offset=_odd_layer_offset(0), arbitrary_size=arbitrary_size,
+                                 wrapped=wrapped)
         self.dw2 = oriented_conv(dim1, kernel_size, stride=2, padding=pad, nhwc=True,
-                                 layer_offset=_odd_layer_offset(1), arbitrary_size=arbitrary_size)
+                                 layer_offset=_odd_layer_offset(1), arbitrary_size=arbitrary_size,
+                                 wrapped=wrapped)
         self.norm1 = nn.LayerNorm(dim1, eps=1e-6)
         self.norm2 = nn.LayerNorm(dim1, eps=1e-6)
         self.norm3 = nn.LayerNorm(dim2, eps=1e-6)
@@ -103,7 +123,7 @@ class Block(nn.Module):
     oriented conv with a residual tap on the 4*dim hidden tensor in NHWC, :322-399)."""
 
     def __init__(self, dim, kernel_sizes, plus_plus, drop_path=0.0, layer_scale_init_value=1e-6,
-                 layer_offset=0.0, n_dir=8, arbitrary_size=False):
+                 layer_offset=0.0, n_dir=8, arbitrary_size=False, wrapped=False):
         super().__init__()
         self.norm = nn.LayerNorm(dim, eps=1e-6)
         self.pwconv1 = nn.Linear(dim, 4 * dim)
@@ -112,12 +132,12 @@ class Block(nn.Module):
                       if layer_scale_init_value > 0 else None)
         self.drop_path = StochasticDepth(drop_path) if drop_path > 0.0 else nn.Identity()
         first = oriented_conv(dim, kernel_sizes[0], n_dir=n_dir, layer_offset=layer_offset,
-                              arbitrary_size=arbitrary_size)
+                              arbitrary_size=arbitrary_size, wrapped=wrapped)
         if plus_plus:
             self.dwconv1 = first
             self.dwconv2 = oriented_conv(4 * dim, kernel_sizes[1], n_dir=n_dir, nhwc=True,
                                          resid=True, layer_offset=layer_offset,
-                                         arbitrary_size=arbitrary_size)
+                                         arbitrary_size=arbitrary_size, wrapped=wrapped)
         else:
             self.dwconv = first
         self.plus_plus = plus_plus
@@ -137,18 +157,23 @@ class Block(nn.Module):
 class ConvNeXt1D(nn.Module):
     """``variant`` "1d" or "1dpp"; ``out_stages=True`` returns the four stage outputs, each
     through its own LayerNorm, instead of logits (the dense-prediction backbone form of
-    semantic_segmentation/backbone/convnext.py:395-399,433-443)."""
+    semantic_segmentation/backbone/convnext.py:395-399,433-443).  ``backbone=True`` is that
+    backbone in full: stage outputs, kernel sizes cropped per stage (:316-327), any input size,
+    and the operators held in wrappers (parameter names ``...dwconv.conv.weight``), so that
+    checkpoints converted by ``backbone_weights.convert_to_backbone_state_dict`` load."""
 
     def __init__(self, in_chans=3, num_classes=1000, depths=(3, 3, 9, 3), dims=(96, 192, 384, 768),
                  drop_path_rate=0.0, layer_scale_init_value=1e-6, head_init_scale=1.0, variant="1d",
-                 N=8, stem_dim1=64, arbitrary_size=False, out_stages=False):
+                 N=8, stem_dim1=64, arbitrary_size=False, out_stages=False, backbone=False):
         super().__init__()
         if variant not in _VARIANTS:
             raise ValueError("variant must be '1d' or '1dpp'")
         block_ks, stem_k = _VARIANTS[variant]
+        stage_ks = _BACKBONE_BLOCK_SIZES[variant] if backbone else (block_ks,) * 4
+        out_stages = out_stages or backbone
         self.out_stages = out_stages
         self.downsample_layers = nn.ModuleList(
-            [Stem1D(in_chans, stem_dim1, dims[0], stem_k, arbitrary_size)])
+            [Stem1D(in_chans, stem_dim1, dims[0], stem_k, arbitrary_size, wrapped=backbone)])
         for i in range(3):
             self.downsample_layers.append(nn.Sequential(
                 ChannelsFirstLayerNorm(dims[i]), nn.Conv2d(dims[i], dims[i + 1], kernel_size=2, stride=2)))
@@ -157,8 +182,9 @@ class ConvNeXt1D(nn.Module):
         done = 0
         for i, depth in enumerate(depths):
             self.stages.append(nn.Sequential(*[
-                Block(dims[i], block_ks, variant == "1dpp", rates[done + j], layer_scale_init_value,
-                      _odd_layer_offset(j), N, arbitrary_size) for j in range(depth)]))
+                Block(dims[i], stage_ks[i], variant == "1dpp", rates[done + j],
+                      layer_scale_init_value, _odd_layer_offset(j), N, arbitrary_size,
+                      wrapped=backbone) for j in range(depth)]))
             done += depth
         if out_stages:
             for i in range(4):

@@ -252,9 +252,12 @@ struct Tile {
     static constexpr int LV = LH, LD = LH;
     static constexpr int PB = 1, NT = 256;
 };
+#ifndef DWO_LH56
+#define DWO_LH56 4
+#endif
 template <>
 struct Tile<56, 56> {  // 784 / 448 / 448 items per plane
-    static constexpr int LH = 4, LV = 7, LD = 8, PB = 1, NT = 448;
+    static constexpr int LH = DWO_LH56, LV = 7, LD = 8, PB = 1, NT = 448;
 };
 template <>
 #ifndef DWO_NTS

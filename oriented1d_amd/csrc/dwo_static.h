@@ -425,6 +425,37 @@ struct ChannelTaps {
     }
 };
 
+// Phase timing for experiments (only with -DDWO_PHASE_TIMING; the product build has none of it):
+// thread 0 of every workgroup accumulates the cycles between consecutive marks per phase id.
+#ifdef DWO_PHASE_TIMING
+__device__ unsigned long long dwo_phase_cycles[4096][8];
+#define DWO_PHASE_MARK(id)                                                   \
+    do {                                                                     \
+        if (threadIdx.x == 0) {                                              \
+            const unsigned long long now_ = __builtin_readcyclecounter();   \
+            if (ph_last_ != 0) ph_acc_[ph_id_] += now_ - ph_last_;          \
+            ph_last_ = now_;                                                 \
+            ph_id_ = id;                                                     \
+        }                                                                    \
+    } while (0)
+#define DWO_PHASE_DONE(o)                                                    \
+    do {                                                                     \
+        if (threadIdx.x == 0 && blockIdx.x < 4096) {                         \
+            for (int i_ = 0; i_ < 6; i_++) dwo_phase_cycles[blockIdx.x][i_] = ph_acc_[i_]; \
+            dwo_phase_cycles[blockIdx.x][6] = o;                             \
+            dwo_phase_cycles[blockIdx.x][7] = __builtin_readcyclecounter() - ph_start_;  \
+        }                                                                    \
+    } while (0)
+#define DWO_PHASE_DECL                                                       \
+    unsigned long long ph_acc_[6] = {0, 0, 0, 0, 0, 0}, ph_last_ = 0;        \
+    const unsigned long long ph_start_ = __builtin_readcyclecounter();       \
+    int ph_id_ = 0;
+#else
+#define DWO_PHASE_MARK(id)
+#define DWO_PHASE_DONE(o)
+#define DWO_PHASE_DECL
+#endif
+
 // ---------------------------------------------------------------------------------------------
 // canonical body
 // ---------------------------------------------------------------------------------------------
@@ -455,6 +486,7 @@ __device__ __forceinline__ void run_canonical(const T *__restrict__ src, const f
     const unsigned tid = threadIdx.x;
     const unsigned pstride = (unsigned)C * (H * W);  // elements between images of one channel
 
+    DWO_PHASE_DECL
     ChannelTaps<G, OP, T, K, PAIR> taps;
     taps.load(wt, bias, c);
 
@@ -470,7 +502,9 @@ __device__ __forceinline__ void run_canonical(const T *__restrict__ src, const f
     // Two register sets keep two batches in flight from HBM while a third is being computed.
     auto process = [&](auto &stg, int nb) {
         const int nvalid = n1 - nb;
+        DWO_PHASE_MARK(0);
         __syncthreads();  // previous batch fully consumed (first pass: zero fill done)
+        DWO_PHASE_MARK(1);
         if constexpr (TILE) {
             if (nb > n0)
                 flush_out_tile<T, H, W, PB, NT>(lout, dbase + (size_t)(nb - PB) * pstride, pstride, PB);
@@ -479,7 +513,9 @@ __device__ __forceinline__ void run_canonical(const T *__restrict__ src, const f
             stg.template commit_pairs<GeoMap<G>, PLS, G::EH, G::EW>(lds, nvalid);
         else
             stg.template commit<GeoMap<G>, PLS>(lds, nvalid);
+        DWO_PHASE_MARK(2);
         __syncthreads();
+        DWO_PHASE_MARK(3);
         if (nb + 2 * PB < n1)
             stg.prefetch(sbase + (size_t)(nb + 2 * PB) * pstride, pstride, n1 - nb - 2 * PB);
         T *obase = dbase + (size_t)nb * pstride;  // uniform
@@ -494,10 +530,13 @@ __device__ __forceinline__ void run_canonical(const T *__restrict__ src, const f
                 taps.accumulate(base, acc);
                 if constexpr (G::CLS == CLS_H) {
                     T *o = obase + (pl * pstride + rb * W + j * L);
-                    if constexpr (L == 4) {
-                        Vec4<T> r;
-                        r.set(acc[0], acc[1], acc[2], acc[3]);
-                        r.store(o);
+                    if constexpr (L % 4 == 0) {
+#pragma unroll
+                        for (int l = 0; l < L; l += 4) {
+                            Vec4<T> r;
+                            r.set(acc[l], acc[l + 1], acc[l + 2], acc[l + 3]);
+                            r.store(o + l);
+                        }
                     } else {
 #pragma unroll
                         for (int l = 0; l < L; l++) st_out(o + l, from_float<T>(acc[l]));
@@ -530,12 +569,15 @@ __device__ __forceinline__ void run_canonical(const T *__restrict__ src, const f
                 }
             }
         }
+        DWO_PHASE_MARK(5);
     };
     int nb = n0;
     for (; nb < n1; nb += 2 * PB) {
         process(sg.a, nb);
         if (nb + PB < n1) process(sg.b, nb + PB);
     }
+    DWO_PHASE_MARK(0);
+    DWO_PHASE_DONE(O);
     if constexpr (TILE) {
         const int last = n0 + ((n1 - n0 - 1) / PB) * PB;  // first image of the final batch
         __syncthreads();
@@ -848,6 +890,16 @@ __global__ __launch_bounds__((Tile<H, W>::NT)) __attribute__((amdgpu_waves_per_e
         run_canonical<O, OP, T, K, H, W>(src, wt, bias, dst, lds, c, C, n0, n1, sg);  \
         break;
     switch (cls) {
+#ifdef DWO_SWITCH_REV
+        DWO_CASE(7)
+        DWO_CASE(6)
+        DWO_CASE(5)
+        DWO_CASE(4)
+        DWO_CASE(3)
+        DWO_CASE(2)
+        DWO_CASE(1)
+        DWO_CASE(0)
+#else
         DWO_CASE(0)
         DWO_CASE(1)
         DWO_CASE(2)
@@ -856,6 +908,7 @@ __global__ __launch_bounds__((Tile<H, W>::NT)) __attribute__((amdgpu_waves_per_e
         DWO_CASE(5)
         DWO_CASE(6)
         DWO_CASE(7)
+#endif
         default:
             run_table<OP, T, K, H, W>(src, wt, bias, taps_dhdw(blob), dst, lds, c, C, n0, n1, sg);
     }

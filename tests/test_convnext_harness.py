@@ -42,6 +42,53 @@ def test_state_dict_layout_and_angles():
     assert m.stages[0][0].dwconv2.resid is not None and m.downsample_layers[0].dw1.stride == (2, 2)
 
 
+@pytest.mark.parametrize("variant", ["1d", "1dpp"])
+def test_backbone_form_and_checkpoint_conversion(variant):
+    """Backbone form: wrapped operator names, per-stage cropped kernels
+    (semantic_segmentation/backbone/convnext.py:74-80,316-327), and the converter: every tensor of
+    the classification checkpoint arrives under its wrapped name, kernels are cropped around the
+    centre tap (the cropped operator equals the original restricted to its inner taps)."""
+    from oriented1d_amd.backbone_weights import centre_crop_kernel, convert_to_backbone_state_dict
+
+    torch.manual_seed(1)
+    cls = ConvNeXt1D(depths=(1, 1, 1, 1), dims=(8, 16, 24, 32), variant=variant, stem_dim1=8,
+                     num_classes=5)
+    bb = ConvNeXt1D(depths=(1, 1, 1, 1), dims=(8, 16, 24, 32), variant=variant, stem_dim1=8,
+                    backbone=True)
+    want = {"1d": [(31,), (31,), (27,), (13,)], "1dpp": [(15, 31), (15, 31), (15, 27), (13, 13)]}[variant]
+    for i in range(4):
+        blk = bb.stages[i][0]
+        convs = [blk.dwconv1, blk.dwconv2] if variant == "1dpp" else [blk.dwconv]
+        assert tuple(c.conv.kernel_size[1] for c in convs) == want[i]
+        assert all(c.conv.arbitrary_size for c in convs)
+    conv = convert_to_backbone_state_dict(cls.state_dict(), bb.state_dict())
+    missing, unexpected = bb.load_state_dict(conv, strict=False)
+    assert not unexpected
+    assert all(k.startswith("norm") for k in missing), missing  # the four per-stage output norms
+    src = cls.state_dict()
+    last = "stages.3.0.dwconv2" if variant == "1dpp" else "stages.3.0.dwconv"
+    w_src, w_dst = src[last + ".weight"], bb.state_dict()[last + ".conv.weight"]
+    K, k = w_src.shape[-1], w_dst.shape[-1]
+    assert k == 13 and torch.equal(w_dst, w_src[..., (K - k) // 2:(K + k) // 2])
+    assert torch.equal(bb.state_dict()[last + ".conv.theta"], src[last + ".theta"])
+    assert torch.equal(bb.state_dict()["stages.0.0.pwconv1.weight"], src["stages.0.0.pwconv1.weight"])
+    w = torch.arange(2 * 7, dtype=torch.float32).reshape(2, 1, 1, 7)
+    assert centre_crop_kernel(w, 3)[0, 0, 0].tolist() == [2.0, 3.0, 4.0]
+    with pytest.raises(ValueError):
+        centre_crop_kernel(w, 4)
+
+
+@pytest.mark.gpu
+def test_backbone_runs_on_odd_input_sizes():
+    torch.manual_seed(0)
+    m = ConvNeXt1D(depths=(1, 1, 1, 1), dims=(8, 16, 24, 32), variant="1d", stem_dim1=8,
+                   backbone=True).cuda().eval()
+    with torch.no_grad():
+        outs = m(torch.randn(1, 3, 72, 104, device="cuda"))
+    assert [tuple(o.shape) for o in outs] == [(1, 8, 18, 26), (1, 16, 9, 13), (1, 24, 4, 6), (1, 32, 2, 3)]
+    assert all(torch.isfinite(o).all() for o in outs)
+
+
 @pytest.mark.gpu
 @pytest.mark.parametrize("variant", ["1d", "1dpp"])
 def test_network_matches_oracle_composition(oracle, variant):
