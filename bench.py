@@ -51,6 +51,9 @@ def main():
                     help="back-to-back launches per (shape, op) for the per-kernel timings")
     ap.add_argument("--kernel-repeats", type=int, default=7,
                     help="repeats of the per-kernel measurement (the median is reported)")
+    ap.add_argument("--no-graph", dest="graph", action="store_false",
+                    help="time eager launches of the 12 C-ABI calls instead of replays of their "
+                         "captured graph")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra-sweeps", action="store_true",
                     help="skip the bf16 / NHWC / grouped-angle rows (other_configs)")
@@ -80,7 +83,10 @@ def main():
 
     from oriented1d_amd import _lib
     lib = _lib.load()
-    stream = torch.cuda.current_stream(dev)
+    # everything runs on one side stream: its handle is what the C ABI launches on, what the
+    # timing events are recorded on, and what the step graphs are captured from
+    stream = torch.cuda.Stream(dev)
+    torch.cuda.set_stream(stream)
     stream_h = ctypes.c_void_p(stream.cuda_stream)
 
     def theta_for(C, kind):
@@ -144,7 +150,7 @@ def main():
 
         step_bytes = sum(algorithmic_bytes(o, BATCH, C, HW, HW, KSIZE, b)
                          for C, HW in STAGES for o in ("fprop", "dgrad", "wgrad"))
-        ms_per_step = None
+        ms_per_step, ms_eager = None, None
         if steps > 0:
             for i in range(warmup):
                 step(i)
@@ -153,7 +159,26 @@ def main():
             for i in range(steps):
                 step(i)
             torch.cuda.synchronize()
-            ms_per_step = (time.perf_counter() - t0) * 1e3 / steps
+            ms_eager = (time.perf_counter() - t0) * 1e3 / steps
+            ms_per_step = ms_eager
+            if args.graph:
+                # the same 12 C-ABI calls per step, captured once per buffer set and replayed:
+                # one launch per step instead of 16 kernel launches from the host
+                graphs = []
+                for i in range(nsets):
+                    gr = torch.cuda.CUDAGraph()
+                    with torch.cuda.graph(gr, stream=stream):
+                        step(i)
+                    graphs.append(gr)
+                for i in range(warmup):
+                    graphs[i % nsets].replay()
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                for i in range(steps):
+                    graphs[i % nsets].replay()
+                torch.cuda.synchronize()
+                ms_per_step = (time.perf_counter() - t0) * 1e3 / steps
+                del graphs
 
         # per-kernel timings: HIP events on the launch stream (torch's current stream is the
         # one passed to the C ABI), median over the repeats
@@ -186,13 +211,15 @@ def main():
                 if warm:
                     detail[key]["warm_us"] = round(timed(name, si, True), 2)
         copy_src = keep[0]
-        res = {"ms_per_step": ms_per_step, "detail": detail, "nsets": nsets,
+        res = {"ms_per_step": ms_per_step, "ms_per_step_eager": ms_eager, "detail": detail,
+               "nsets": nsets,
                "step_bytes": step_bytes, "copy_src": copy_src if args.calibration_copy else None}
         return res
 
     main_res = sweep(args.dtype, args.layout, args.theta, args.steps, args.warmup,
                      args.kernel_iters, args.kernel_repeats, args.only, warm=True)
     ms_per_step, detail = main_res["ms_per_step"], main_res["detail"]
+    main_res_eager = main_res["ms_per_step_eager"]
     nsets, step_bytes = main_res["nsets"], main_res["step_bytes"]
     value = step_bytes / (ms_per_step * 1e-3) / 1e9
 
@@ -350,6 +377,9 @@ def main():
                                "(C=96@56x56, 192@28x28, 384@14x14, 768@7x7), batch 64, K=31, "
                                "8 orientations %s, stride 1" % args.theta,
                    "layout": args.layout, "buffer_sets": nsets,
+                   "launch": ("hipGraph replay of the step's 12 C-ABI calls (one graph per "
+                              "buffer set)" if args.graph else "eager C-ABI calls"),
+                   "ms_per_step_eager": round(main_res_eager, 4),
                    "algorithmic_bytes_per_step": step_bytes},
         "frac_hbm_peak": round(value / HBM_PEAK_GBS, 4),
         "detail": detail, "roofline": roofline, "cpu_baseline": cpu,

@@ -13,10 +13,3 @@ template int launch_nhwc_plane_conv<DWO_INST_T, DWO_INST_K, DWO_INST_H, DWO_INST
 template int launch_nhwc_plane_wgrad<DWO_INST_T, DWO_INST_K, DWO_INST_H, DWO_INST_W>(
     const void *, const void *, const void *, float *, int, int, int *, hipStream_t);
 }  // namespace dwo
-
-
-#ifdef DWO_PHASE_TIMING
-extern "C" int dwo_debug_phase_read(void *host, size_t bytes) {
-    return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(dwo::dwo_phase_cycles), bytes);
-}
-#endif

@@ -252,36 +252,21 @@ struct Tile {
     static constexpr int LV = LH, LD = LH;
     static constexpr int PB = 1, NT = 256;
 };
-#ifndef DWO_LH56
-#define DWO_LH56 4
-#endif
 template <>
 struct Tile<56, 56> {  // 784 / 448 / 448 items per plane
-    static constexpr int LH = DWO_LH56, LV = 7, LD = 8, PB = 1, NT = 448;
+    static constexpr int LH = 4, LV = 7, LD = 8, PB = 1, NT = 448;
 };
 template <>
-#ifndef DWO_NTS
-#define DWO_NTS 448
-#endif
-#ifndef DWO_PB28
-#define DWO_PB28 2
-#endif
-#ifndef DWO_PB14
-#define DWO_PB14 4
-#endif
-#ifndef DWO_PB7
-#define DWO_PB7 8
-#endif
 struct Tile<28, 28> {  // 196 / 196 / 224
-    static constexpr int LH = 4, LV = 4, LD = 4, PB = DWO_PB28, NT = DWO_NTS;
+    static constexpr int LH = 4, LV = 4, LD = 4, PB = 2, NT = 448;
 };
 template <>
 struct Tile<14, 14> {  // 98 / 98 / 112
-    static constexpr int LH = 2, LV = 2, LD = 2, PB = DWO_PB14, NT = DWO_NTS;
+    static constexpr int LH = 2, LV = 2, LD = 2, PB = 4, NT = 448;
 };
 template <>
 struct Tile<7, 7> {  // 49 / 49 / 56
-    static constexpr int LH = 1, LV = 1, LD = 1, PB = DWO_PB7, NT = DWO_NTS;
+    static constexpr int LH = 1, LV = 1, LD = 1, PB = 8, NT = 448;
 };
 template <int H, int W>
 constexpr int tile_L(int o) {

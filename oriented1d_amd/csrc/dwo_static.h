@@ -8,12 +8,10 @@
 // the table-driven body at the bottom (same staging, dynamic taps).
 #pragma once
 
-#ifndef DWO_WPE
+// Register budget of the plane kernels: at least six waves per SIMD, i.e. three 448-thread
+// workgroups per CU (seven would need 72 registers and spill).
 #define DWO_WPE 6
-#endif
-#ifndef DWO_WPE_WGRAD
 #define DWO_WPE_WGRAD 6
-#endif
 
 #include "dwo_common.h"
 #include "dwo_dispatch.h"
@@ -425,37 +423,6 @@ struct ChannelTaps {
     }
 };
 
-// Phase timing for experiments (only with -DDWO_PHASE_TIMING; the product build has none of it):
-// thread 0 of every workgroup accumulates the cycles between consecutive marks per phase id.
-#ifdef DWO_PHASE_TIMING
-__device__ unsigned long long dwo_phase_cycles[4096][8];
-#define DWO_PHASE_MARK(id)                                                   \
-    do {                                                                     \
-        if (threadIdx.x == 0) {                                              \
-            const unsigned long long now_ = __builtin_readcyclecounter();   \
-            if (ph_last_ != 0) ph_acc_[ph_id_] += now_ - ph_last_;          \
-            ph_last_ = now_;                                                 \
-            ph_id_ = id;                                                     \
-        }                                                                    \
-    } while (0)
-#define DWO_PHASE_DONE(o)                                                    \
-    do {                                                                     \
-        if (threadIdx.x == 0 && blockIdx.x < 4096) {                         \
-            for (int i_ = 0; i_ < 6; i_++) dwo_phase_cycles[blockIdx.x][i_] = ph_acc_[i_]; \
-            dwo_phase_cycles[blockIdx.x][6] = o;                             \
-            dwo_phase_cycles[blockIdx.x][7] = __builtin_readcyclecounter() - ph_start_;  \
-        }                                                                    \
-    } while (0)
-#define DWO_PHASE_DECL                                                       \
-    unsigned long long ph_acc_[6] = {0, 0, 0, 0, 0, 0}, ph_last_ = 0;        \
-    const unsigned long long ph_start_ = __builtin_readcyclecounter();       \
-    int ph_id_ = 0;
-#else
-#define DWO_PHASE_MARK(id)
-#define DWO_PHASE_DONE(o)
-#define DWO_PHASE_DECL
-#endif
-
 // ---------------------------------------------------------------------------------------------
 // canonical body
 // ---------------------------------------------------------------------------------------------
@@ -466,11 +433,7 @@ __device__ unsigned long long dwo_phase_cycles[4096][8];
 // words leave a thread as whole 32-bit writes) on planes whose rows split into 4-element chunks.
 template <typename T, int O, int W>
 constexpr bool use_pairs() {
-#ifdef DWO_NO_PAIRS
-    return false;
-#else
     return sizeof(T) == 2 && orient_class(O) == CLS_H && W % 4 == 0;
-#endif
 }
 template <int O, int OP, typename T, int K, int H, int W>
 __device__ __forceinline__ void run_canonical(const T *__restrict__ src, const float *__restrict__ wt,
@@ -486,7 +449,6 @@ __device__ __forceinline__ void run_canonical(const T *__restrict__ src, const f
     const unsigned tid = threadIdx.x;
     const unsigned pstride = (unsigned)C * (H * W);  // elements between images of one channel
 
-    DWO_PHASE_DECL
     ChannelTaps<G, OP, T, K, PAIR> taps;
     taps.load(wt, bias, c);
 
@@ -502,9 +464,7 @@ __device__ __forceinline__ void run_canonical(const T *__restrict__ src, const f
     // Two register sets keep two batches in flight from HBM while a third is being computed.
     auto process = [&](auto &stg, int nb) {
         const int nvalid = n1 - nb;
-        DWO_PHASE_MARK(0);
         __syncthreads();  // previous batch fully consumed (first pass: zero fill done)
-        DWO_PHASE_MARK(1);
         if constexpr (TILE) {
             if (nb > n0)
                 flush_out_tile<T, H, W, PB, NT>(lout, dbase + (size_t)(nb - PB) * pstride, pstride, PB);
@@ -513,9 +473,7 @@ __device__ __forceinline__ void run_canonical(const T *__restrict__ src, const f
             stg.template commit_pairs<GeoMap<G>, PLS, G::EH, G::EW>(lds, nvalid);
         else
             stg.template commit<GeoMap<G>, PLS>(lds, nvalid);
-        DWO_PHASE_MARK(2);
         __syncthreads();
-        DWO_PHASE_MARK(3);
         if (nb + 2 * PB < n1)
             stg.prefetch(sbase + (size_t)(nb + 2 * PB) * pstride, pstride, n1 - nb - 2 * PB);
         T *obase = dbase + (size_t)nb * pstride;  // uniform
@@ -569,15 +527,12 @@ __device__ __forceinline__ void run_canonical(const T *__restrict__ src, const f
                 }
             }
         }
-        DWO_PHASE_MARK(5);
     };
     int nb = n0;
     for (; nb < n1; nb += 2 * PB) {
         process(sg.a, nb);
         if (nb + PB < n1) process(sg.b, nb + PB);
     }
-    DWO_PHASE_MARK(0);
-    DWO_PHASE_DONE(O);
     if constexpr (TILE) {
         const int last = n0 + ((n1 - n0 - 1) / PB) * PB;  // first image of the final batch
         __syncthreads();
@@ -890,16 +845,6 @@ __global__ __launch_bounds__((Tile<H, W>::NT)) __attribute__((amdgpu_waves_per_e
         run_canonical<O, OP, T, K, H, W>(src, wt, bias, dst, lds, c, C, n0, n1, sg);  \
         break;
     switch (cls) {
-#ifdef DWO_SWITCH_REV
-        DWO_CASE(7)
-        DWO_CASE(6)
-        DWO_CASE(5)
-        DWO_CASE(4)
-        DWO_CASE(3)
-        DWO_CASE(2)
-        DWO_CASE(1)
-        DWO_CASE(0)
-#else
         DWO_CASE(0)
         DWO_CASE(1)
         DWO_CASE(2)
@@ -908,7 +853,6 @@ __global__ __launch_bounds__((Tile<H, W>::NT)) __attribute__((amdgpu_waves_per_e
         DWO_CASE(5)
         DWO_CASE(6)
         DWO_CASE(7)
-#endif
         default:
             run_table<OP, T, K, H, W>(src, wt, bias, taps_dhdw(blob), dst, lds, c, C, n0, n1, sg);
     }
