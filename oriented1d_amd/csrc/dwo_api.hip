@@ -83,11 +83,11 @@ int try_plane_conv(int op, const void *src, const float *w, const float *bias, c
 }
 
 template <typename T>
-int try_plane_wgrad(const void *x, const void *dy, const void *taps, float *part, int *groups,
-                    const ConvDims &d, hipStream_t st) {
+int try_plane_wgrad(const void *x, const void *dy, const void *taps, float *part, float *dw,
+                    float *db, int *groups, const ConvDims &d, hipStream_t st) {
 #define DWO_MATCH(K_, H_, W_)                                                               \
     if (d.K == K_ && d.H == H_ && d.W == W_)                                                \
-        return launch_plane_wgrad<T, K_, H_, W_>(x, dy, taps, part, d.N, d.C, groups, st);
+        return launch_plane_wgrad<T, K_, H_, W_>(x, dy, taps, part, dw, db, d.N, d.C, groups, st);
     DWO_PLANE_SHAPES(DWO_MATCH)
 #undef DWO_MATCH
     return -100;
@@ -129,11 +129,12 @@ int nhwc_plane_batch(const ConvDims &d, int layout) {
 }
 
 template <typename T>
-int try_nhwc_plane_wgrad(const void *x, const void *dy, const void *taps, float *part, int *groups,
-                         const ConvDims &d, hipStream_t st) {
+int try_nhwc_plane_wgrad(const void *x, const void *dy, const void *taps, float *part, float *dw,
+                         float *db, int *groups, const ConvDims &d, hipStream_t st) {
 #define DWO_MATCH(K_, H_, W_)                                                                    \
     if (d.K == K_ && d.H == H_ && d.W == W_)                                                     \
-        return launch_nhwc_plane_wgrad<T, K_, H_, W_>(x, dy, taps, part, d.N, d.C, groups, st);
+        return launch_nhwc_plane_wgrad<T, K_, H_, W_>(x, dy, taps, part, dw, db, d.N, d.C, groups, \
+                                                      st);
     DWO_PLANE_SHAPES(DWO_MATCH)
 #undef DWO_MATCH
     return -100;
@@ -248,10 +249,13 @@ int wgrad_t(const void *dy, const void *x, const void *taps, float *dw, float *d
             const ConvDims &d, int layout, hipStream_t st) {
     float *part = (float *)scratch;
     int rc, NG = 0;
+    bool direct = false;  // a single group per channel: stage 1 wrote dw / db itself
     if (plane_batch(d, layout) != 0) {
-        rc = try_plane_wgrad<T>(x, dy, taps, part, &NG, d, st);
+        rc = try_plane_wgrad<T>(x, dy, taps, part, dw, db, &NG, d, st);
+        direct = NG == 1;
     } else if (nhwc_plane_batch(d, layout) != 0) {
-        rc = try_nhwc_plane_wgrad<T>(x, dy, taps, part, &NG, d, st);
+        rc = try_nhwc_plane_wgrad<T>(x, dy, taps, part, dw, db, &NG, d, st);
+        direct = NG == 1;
     } else if (layout == DWO_NHWC && nhwc_has_k(d.K)) {
         rc = try_nhwc_wgrad<T>(dy, x, taps, part, &NG, d, st);
     } else {
@@ -267,7 +271,7 @@ int wgrad_t(const void *dy, const void *x, const void *taps, float *dw, float *d
                 (const T *)dy, (const T *)x, tp, part, d, s.G, s.per_slice);
         rc = launch_status();
     }
-    if (rc != DWO_OK) return rc;
+    if (rc != DWO_OK || direct) return rc;
     const int cells = d.C * (d.K + 1);
     wgrad_reduce_kernel<<<dim3((cells + 255) / 256), dim3(256), 0, st>>>(part, dw, db, d.C, d.K,
                                                                         NG);

@@ -417,12 +417,12 @@ struct NhwcWgradCtx : NhwcCtx<T, K, H, W> {
     }
 };
 
-// Sub-group epilogue: per-thread accumulators -> wave totals (DPP) -> LDS -> one partial per
-// value written to part[(c*(K+1) + s) * NG + group].
+// Sub-group epilogue: per-thread accumulators -> wave totals (DPP) -> LDS -> one value per tap
+// handed to WgradOut.
 template <int K, int NT, int NTS, class SlotOf>
 __device__ __forceinline__ void wgrad_epilogue_sub(float (&acc)[K + 1], float *lds,
-                                                   float *__restrict__ part, int c, int sub,
-                                                   unsigned stid, int group, int NG, SlotOf slot_of) {
+                                                   const WgradOut &out, int c, int sub,
+                                                   unsigned stid, int group, SlotOf slot_of) {
     constexpr int NWS = NTS / 64;
     __syncthreads();  // staged planes are dead from here on
 #pragma unroll
@@ -436,15 +436,15 @@ __device__ __forceinline__ void wgrad_epilogue_sub(float (&acc)[K + 1], float *l
         float t = 0.f;
         if (slot >= 0)
             for (int w = 0; w < NWS; w++) t += lds[(sub * NWS + w) * (K + 1) + slot];
-        part[((size_t)c * (K + 1) + stid) * NG + group] = t;
+        out.put(c, (int)stid, group, K, t);
     }
 }
 
 // Barriers per batch are the same in every body: two per phase.
 template <int O, typename T, int K, int H, int W>
 __device__ __forceinline__ void nhwc_canonical_wgrad(NhwcWgradCtx<T, K, H, W> &ctx,
-                                                     float *__restrict__ part, int c, int sub,
-                                                     unsigned stid, int n0, int group, int NG) {
+                                                     const WgradOut &out, int c, int sub,
+                                                     unsigned stid, int n0, int group) {
     using Ctx = NhwcWgradCtx<T, K, H, W>;
     constexpr int L = tile_L<H, W>(O);
     constexpr int PBI = Ctx::PBI, NT = Ctx::NT, NTS = NT / kSliceCh, PLS = Ctx::PLS, DYP = Ctx::DYP;
@@ -517,15 +517,15 @@ __device__ __forceinline__ void nhwc_canonical_wgrad(NhwcWgradCtx<T, K, H, W> &c
             __syncthreads();  // staged x and dy of this phase are consumed
         });
     }
-    wgrad_epilogue_sub<K, NT, NTS>(acc, ctx.lds, part, c, sub, stid, group, NG,
+    wgrad_epilogue_sub<K, NT, NTS>(acc, ctx.lds, out, c, sub, stid, group,
                                    [](int s) { return (int)G::plan.rep[s]; });
 }
 
 template <typename T, int K, int H, int W>
 __device__ __forceinline__ void nhwc_table_wgrad(NhwcWgradCtx<T, K, H, W> &ctx,
                                                  const int8_t *__restrict__ dhdw,
-                                                 float *__restrict__ part, int c, int sub,
-                                                 unsigned stid, int n0, int group, int NG) {
+                                                 const WgradOut &out, int c, int sub,
+                                                 unsigned stid, int n0, int group) {
     using Ctx = NhwcWgradCtx<T, K, H, W>;
     using Map = TableMap<K, H, W>;
     constexpr int PBI = Ctx::PBI, NT = Ctx::NT, NTS = NT / kSliceCh, PLS = Ctx::PLS, DYP = Ctx::DYP;
@@ -573,16 +573,17 @@ __device__ __forceinline__ void nhwc_table_wgrad(NhwcWgradCtx<T, K, H, W> &ctx,
             __syncthreads();
         });
     }
-    wgrad_epilogue_sub<K, NT, NTS>(acc, ctx.lds, part, c, sub, stid, group, NG,
+    wgrad_epilogue_sub<K, NT, NTS>(acc, ctx.lds, out, c, sub, stid, group,
                                    [&](int s) { return tlive[s]; });
 }
 
 template <typename T, int K, int H, int W>
 __global__ __launch_bounds__((NhwcTile<H, W>::NT)) void nhwc_plane_wgrad_kernel(
     const T *__restrict__ x, const T *__restrict__ dy, const void *__restrict__ blob,
-    float *__restrict__ part, int N, int C, int NG) {
+    WgradOut out, int N, int C) {
     extern __shared__ float lds[];
     using Ctx = NhwcWgradCtx<T, K, H, W>;
+    const int NG = out.NG;
     constexpr int NTS = Ctx::NT / kSliceCh;
     int slice, group;
     nhwc_task(C / kSliceCh, NG, 128 / (kSliceCh * (int)sizeof(T)), slice, group);
@@ -608,7 +609,7 @@ __global__ __launch_bounds__((NhwcTile<H, W>::NT)) void nhwc_plane_wgrad_kernel(
     const int mine = cls[sub];
 #define DWO_CASE(O)                                                                     \
     case O:                                                                             \
-        nhwc_canonical_wgrad<O, T, K, H, W>(ctx, part, c, sub, stid, n0, group, NG);     \
+        nhwc_canonical_wgrad<O, T, K, H, W>(ctx, out, c, sub, stid, n0, group);          \
         break;
     switch (mine) {
         DWO_CASE(0)
@@ -620,15 +621,15 @@ __global__ __launch_bounds__((NhwcTile<H, W>::NT)) void nhwc_plane_wgrad_kernel(
         DWO_CASE(6)
         DWO_CASE(7)
         default:
-            nhwc_table_wgrad<T, K, H, W>(ctx, taps_dhdw(blob), part, c, sub, stid, n0, group, NG);
+            nhwc_table_wgrad<T, K, H, W>(ctx, taps_dhdw(blob), out, c, sub, stid, n0, group);
     }
 #undef DWO_CASE
 }
 
-// Writes NG = *groups_out partials per (channel, tap) into part[(c*(K+1)+s)*NG + g].
+// Same contract as launch_plane_wgrad.
 template <typename T, int K, int H, int W>
-int launch_nhwc_plane_wgrad(const void *x, const void *dy, const void *taps, float *part, int N,
-                            int C, int *groups_out, hipStream_t st) {
+int launch_nhwc_plane_wgrad(const void *x, const void *dy, const void *taps, float *part, float *dw,
+                            float *db, int N, int C, int *groups_out, hipStream_t st) {
     constexpr int NT = NhwcTile<H, W>::NT, PBI = NhwcTile<H, W>::PBI;
     const size_t lds = nhwc_plane_wgrad_lds_bytes<K, H, W>();
     static const int slots = [&] {
@@ -639,7 +640,7 @@ int launch_nhwc_plane_wgrad(const void *x, const void *dy, const void *taps, flo
     const int groups = plane_groups(N, nslices, PBI, slots);
     *groups_out = groups;
     nhwc_plane_wgrad_kernel<T, K, H, W><<<dim3(nslices * groups), dim3(NT), lds, st>>>(
-        (const T *)x, (const T *)dy, taps, part, N, C, groups);
+        (const T *)x, (const T *)dy, taps, WgradOut{part, dw, db, groups}, N, C);
     const hipError_t e = hipGetLastError();
     return e == hipSuccess ? 0 : (int)e;
 }

@@ -629,11 +629,26 @@ __device__ __forceinline__ float wave_sum_dpp(float v) {
 }
 
 // Workgroup epilogue: per-thread accumulators acc[0..NV) -> wave totals (DPP) -> LDS -> one
-// partial per value written to part[(c*(K+1) + s) * NG + group].  `slot_of(s)` maps tap s to the
+// value per tap handed to WgradOut.  `slot_of(s)` maps tap s to the
 // accumulator that holds its sum (-1: the tap never reaches the plane, its gradient is zero).
+// Where a workgroup's sums go: one partial per (channel, tap, group) in scratch for the stage-2
+// reduction, or, when a channel has a single group, straight into dw / db.
+struct WgradOut {
+    float *part, *dw, *db;
+    int NG;
+    __device__ __forceinline__ void put(int c, int s, int group, int K, float t) const {
+        if (NG > 1)
+            part[((size_t)c * (K + 1) + s) * NG + group] = t;
+        else if (s < K)
+            dw[(size_t)c * K + s] = t;
+        else if (db != nullptr)
+            db[c] = t;
+    }
+};
+
 template <int K, int NT, class SlotOf>
-__device__ __forceinline__ void wgrad_epilogue(float (&acc)[K + 1], float *lds, float *__restrict__ part,
-                                               int c, int group, int NG, SlotOf slot_of) {
+__device__ __forceinline__ void wgrad_epilogue(float (&acc)[K + 1], float *lds, const WgradOut &out,
+                                               int c, int group, SlotOf slot_of) {
     constexpr int NW = NT / 64;
     __syncthreads();  // staged planes are dead from here on
 #pragma unroll
@@ -647,7 +662,7 @@ __device__ __forceinline__ void wgrad_epilogue(float (&acc)[K + 1], float *lds, 
         float t = 0.f;
         if (slot >= 0)
             for (int w = 0; w < NW; w++) t += lds[w * (K + 1) + slot];
-        part[((size_t)c * (K + 1) + threadIdx.x) * NG + group] = t;
+        out.put(c, threadIdx.x, group, K, t);
     }
 }
 
@@ -664,8 +679,8 @@ constexpr int wgrad_dy_offset() {
 
 template <int O, typename T, int K, int H, int W>
 __device__ __forceinline__ void run_canonical_wgrad(const T *__restrict__ x, const T *__restrict__ dy,
-                                                    float *__restrict__ part, float *lds, int c,
-                                                    int C, int n0, int n1, int group, int NG) {
+                                                    const WgradOut &out, float *lds, int c,
+                                                    int C, int n0, int n1, int group) {
     constexpr int L = tile_L<H, W>(O);
     constexpr int PB = Tile<H, W>::PB, NT = Tile<H, W>::NT;
     using G = Geo<O, K, L, H, W>;
@@ -734,16 +749,15 @@ __device__ __forceinline__ void run_canonical_wgrad(const T *__restrict__ x, con
             }
         }
     }
-    wgrad_epilogue<K, NT>(acc, lds, part, c, group, NG,
-                          [](int s) { return (int)G::plan.rep[s]; });
+    wgrad_epilogue<K, NT>(acc, lds, out, c, group, [](int s) { return (int)G::plan.rep[s]; });
 }
 
 // table-driven wgrad body (any angle)
 template <typename T, int K, int H, int W>
 __device__ __forceinline__ void run_table_wgrad(const T *__restrict__ x, const T *__restrict__ dy,
                                                 const int8_t *__restrict__ dhdw,
-                                                float *__restrict__ part, float *lds, int c, int C,
-                                                int n0, int n1, int group, int NG) {
+                                                const WgradOut &out, float *lds, int c, int C,
+                                                int n0, int n1, int group) {
     constexpr int PB = Tile<H, W>::PB, NT = Tile<H, W>::NT;
     using Map = TableMap<K, H, W>;
     constexpr int PLS = plane_floats<K, H, W>();
@@ -785,14 +799,15 @@ __device__ __forceinline__ void run_table_wgrad(const T *__restrict__ x, const T
             acc[K] += gy;
         }
     }
-    wgrad_epilogue<K, NT>(acc, lds, part, c, group, NG, [&](int s) { return tlive[s]; });
+    wgrad_epilogue<K, NT>(acc, lds, out, c, group, [&](int s) { return tlive[s]; });
 }
 
 template <typename T, int K, int H, int W>
 __global__ __launch_bounds__((Tile<H, W>::NT)) __attribute__((amdgpu_waves_per_eu(DWO_WPE_WGRAD, 8))) void plane_wgrad_kernel(
     const T *__restrict__ x, const T *__restrict__ dy, const void *__restrict__ blob,
-    float *__restrict__ part, int N, int C, int NG) {
+    WgradOut out, int N, int C) {
     extern __shared__ float lds[];
+    const int NG = out.NG;
     int c, group;
     plane_task(C, NG, c, group);
     int n0, n1;
@@ -800,7 +815,7 @@ __global__ __launch_bounds__((Tile<H, W>::NT)) __attribute__((amdgpu_waves_per_e
     const int cls = taps_class(blob, C, K)[c];
 #define DWO_CASE(O)                                                                      \
     case O:                                                                              \
-        run_canonical_wgrad<O, T, K, H, W>(x, dy, part, lds, c, C, n0, n1, group, NG);    \
+        run_canonical_wgrad<O, T, K, H, W>(x, dy, out, lds, c, C, n0, n1, group);         \
         break;
     switch (cls) {
         DWO_CASE(0)
@@ -812,7 +827,7 @@ __global__ __launch_bounds__((Tile<H, W>::NT)) __attribute__((amdgpu_waves_per_e
         DWO_CASE(6)
         DWO_CASE(7)
         default:
-            run_table_wgrad<T, K, H, W>(x, dy, taps_dhdw(blob), part, lds, c, C, n0, n1, group, NG);
+            run_table_wgrad<T, K, H, W>(x, dy, taps_dhdw(blob), out, lds, c, C, n0, n1, group);
     }
 #undef DWO_CASE
 }
@@ -892,17 +907,18 @@ int launch_plane_conv(int op, const void *src, const float *w, const float *bias
     return e == hipSuccess ? 0 : (int)e;
 }
 
-// Writes NG = *groups_out partials per (channel, tap) into part[(c*(K+1)+s)*NG + g].
+// Writes NG = *groups_out partials per (channel, tap) into part[(c*(K+1)+s)*NG + g]; with
+// NG = 1 the sums go straight to dw / db (db may be null) and no reduction is needed.
 template <typename T, int K, int H, int W>
-int launch_plane_wgrad(const void *x, const void *dy, const void *taps, float *part, int N, int C,
-                       int *groups_out, hipStream_t st) {
+int launch_plane_wgrad(const void *x, const void *dy, const void *taps, float *part, float *dw,
+                       float *db, int N, int C, int *groups_out, hipStream_t st) {
     constexpr int NT = Tile<H, W>::NT;
     const size_t lds = plane_wgrad_lds_bytes<K, H, W>();
     static const int slots = resident_slots(plane_wgrad_kernel<T, K, H, W>, NT, lds);
     const int groups = plane_groups(N, C, Tile<H, W>::PB, slots);
     *groups_out = groups;
     plane_wgrad_kernel<T, K, H, W><<<dim3(C * groups), dim3(NT), lds, st>>>(
-        (const T *)x, (const T *)dy, taps, part, N, C, groups);
+        (const T *)x, (const T *)dy, taps, WgradOut{part, dw, db, groups}, N, C);
     const hipError_t e = hipGetLastError();
     return e == hipSuccess ? 0 : (int)e;
 }
