@@ -303,7 +303,7 @@ const char *dwo_status_string(int status) {
 
 size_t dwo_taps_bytes(int C, int K) {
     if (C < 1 || K < 1 || K > DWO_MAX_K || (K & 1) == 0) return 0;
-    return kTapsHeaderBytes + taps_dhdw_bytes(C, K) + (((size_t)C * 4 + 15) & ~(size_t)15);
+    return kTapsHeaderBytes + taps_dhdw_bytes(C, K) + 2 * taps_class_bytes(C);
 }
 
 int dwo_build_taps(const float *theta_host, int C, int K, void *taps_host) {
@@ -336,6 +336,20 @@ int dwo_build_taps(const float *theta_host, int C, int K, void *taps_host) {
                 same = dhdw[((size_t)c * K + s) * 2] == canon_dh(o, K, s) &&
                        dhdw[((size_t)c * K + s) * 2 + 1] == canon_dw(o, K, s);
             if (same) cls[c] = o;
+        }
+    }
+    // channel order that cycles through the classes: 0, 1, .., 7, non-canonical, 0, 1, ..
+    hdr[6] = hdr[5] + (int32_t)taps_class_bytes(C);
+    int32_t *order = (int32_t *)((int8_t *)taps_host + hdr[6]);
+    int next[9];  // per class: next channel of that class not yet placed
+    for (int k = 0; k < 9; k++) next[k] = 0;
+    for (int placed = 0; placed < C;) {
+        for (int k = 0; k < 9 && placed < C; k++) {
+            const int want = k < 8 ? k : -1;
+            int c = next[k];
+            while (c < C && cls[c] != want) c++;
+            next[k] = c + 1;
+            if (c < C) order[placed++] = c;
         }
     }
     return DWO_OK;

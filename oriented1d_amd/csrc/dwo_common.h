@@ -10,13 +10,19 @@ namespace dwo {
 
 // ---------------------------------------------------------------------------------------------
 // Tap blob (private layout).  Built on the host by dwo_build_taps, copied verbatim to the device.
-//   int32 header[8] : magic, version, C, K, off_dhdw, off_class, 0, 0
+//   int32 header[8] : magic, version, C, K, off_dhdw, off_class, off_order, 0
 //   int8  dhdw[C][K][2]        (dh, dw) of every tap, padded to 16 bytes
 //   int32 cls[C]               canonical orientation id 0..7 of the channel's tap pattern
-//                              (k * 22.5 degrees), or -1 when the pattern is not canonical
+//                              (k * 22.5 degrees), or -1 when the pattern is not canonical;
+//                              padded to 16 bytes
+//   int32 order[C]             the channels in an order that cycles through the orientation
+//                              classes (class 0, 1, .., 7, other, 0, 1, ..): per-channel
+//                              workgroups take their channel from it, so that whatever way the
+//                              angles are laid out over the channels, neighbouring workgroup
+//                              ids (hence every XCD and CU) get a mix of orientations
 // ---------------------------------------------------------------------------------------------
 constexpr int32_t kTapsMagic = 0x44574f31;  // "DWO1"
-constexpr int32_t kTapsVersion = 2;
+constexpr int32_t kTapsVersion = 3;
 constexpr int kTapsHeaderInts = 8;
 constexpr int kTapsHeaderBytes = kTapsHeaderInts * 4;
 
@@ -26,9 +32,17 @@ __host__ __device__ inline size_t taps_dhdw_bytes(int C, int K) {
 __host__ __device__ inline const int8_t *taps_dhdw(const void *blob) {
     return reinterpret_cast<const int8_t *>(blob) + kTapsHeaderBytes;
 }
+__host__ __device__ inline size_t taps_class_bytes(int C) {
+    return ((size_t)C * 4 + 15) & ~(size_t)15;
+}
 __host__ __device__ inline const int32_t *taps_class(const void *blob, int C, int K) {
     return reinterpret_cast<const int32_t *>(reinterpret_cast<const int8_t *>(blob) +
                                              kTapsHeaderBytes + taps_dhdw_bytes(C, K));
+}
+__host__ __device__ inline const int32_t *taps_order(const void *blob, int C, int K) {
+    return reinterpret_cast<const int32_t *>(reinterpret_cast<const int8_t *>(blob) +
+                                             kTapsHeaderBytes + taps_dhdw_bytes(C, K) +
+                                             taps_class_bytes(C));
 }
 
 // ---------------------------------------------------------------------------------------------

@@ -297,15 +297,17 @@ constexpr int plan_fma_count(const P &p, int L) {
 }
 
 // Workgroup -> (channel, image group).  Hardware hands consecutive workgroup ids to the eight
-// XCDs round-robin and fills the CUs of an XCD in order, while orientation (hence cost) often
-// repeats with period 8 over the channels; rotating the task id inside every aligned block of
-// eight ids by (block + block/32) gives every XCD and every CU a mix of orientations.
-__device__ __forceinline__ void plane_task(int C, int groups, int &c, int &group) {
+// XCDs round-robin and fills the CUs of an XCD in order.  Channels are taken from the tap
+// table's class-cycling order (position p holds a channel of class p mod 8 while all classes
+// last), and the task id is rotated inside every aligned block of eight ids by
+// (block + block/32), so every XCD and every CU gets a mix of orientations (hence of costs).
+__device__ __forceinline__ void plane_task(const void *blob, int C, int K, int groups, int &c,
+                                           int &group) {
     const int i = blockIdx.x, total = C * groups;
     const int j = i >> 3;
     int t = i;
     if (j * 8 + 8 <= total) t = (j << 3) + ((i + j + (j >> 5)) & 7);
-    c = t % C;
+    c = taps_order(blob, C, K)[t % C];
     group = t / C;
 }
 // Images [n0, n1) of group g: the ceil(N/PB) staged batches are split as evenly as possible.
@@ -809,7 +811,7 @@ __global__ __launch_bounds__((Tile<H, W>::NT)) __attribute__((amdgpu_waves_per_e
     extern __shared__ float lds[];
     const int NG = out.NG;
     int c, group;
-    plane_task(C, NG, c, group);
+    plane_task(blob, C, K, NG, c, group);
     int n0, n1;
     group_range<Tile<H, W>::PB>(N, NG, group, n0, n1);
     const int cls = taps_class(blob, C, K)[c];
@@ -849,7 +851,7 @@ __global__ __launch_bounds__((Tile<H, W>::NT)) __attribute__((amdgpu_waves_per_e
     const void *__restrict__ blob, T *__restrict__ dst, int N, int C, int groups) {
     extern __shared__ float lds[];
     int c, group;
-    plane_task(C, groups, c, group);
+    plane_task(blob, C, K, groups, c, group);
     int n0, n1;
     group_range<Tile<H, W>::PB>(N, groups, group, n0, n1);
     ConvStagers<T, H, W> sg;

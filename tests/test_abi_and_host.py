@@ -68,6 +68,29 @@ def test_host_tap_table_equals_oracle(oracle, K):
     assert (dh == odh).all() and (dw == odw).all()
 
 
+@pytest.mark.parametrize("layout", ["grouped", "roundrobin", "mixed"])
+def test_tap_table_channel_order_cycles_through_classes(layout):
+    """The blob's channel order is a permutation of the channels in which, while every class
+    still has channels left, eight consecutive entries hold the eight orientation classes."""
+    from parity_util import canonical_theta, grouped_theta
+    C, K = 96, 31
+    theta = {"grouped": grouped_theta(C), "roundrobin": canonical_theta(C),
+             "mixed": np.concatenate([grouped_theta(64), np.full(32, 0.3, np.float32)])}[layout]
+    blob = op.build_taps(torch.from_numpy(theta.astype(np.float32)), C, K).numpy()
+    hdr = blob[:32].view(np.int32)
+    cls = blob[hdr[5]:hdr[5] + 4 * C].view(np.int32)
+    order = blob[hdr[6]:hdr[6] + 4 * C].view(np.int32)
+    assert sorted(order.tolist()) == list(range(C))
+    if layout != "mixed":
+        assert set(cls.tolist()) == set(range(8))
+        for i in range(0, C, 8):
+            assert sorted(cls[order[i:i + 8]].tolist()) == list(range(8)), i
+    else:
+        assert (cls[64:] == -1).all()
+        first = cls[order[:72]].reshape(8, 9)  # eight full cycles over 8 classes + "other"
+        assert all(sorted(r.tolist()) == [-1] + list(range(8)) for r in first)
+
+
 def test_module_contract():
     C, K = 16, 31
     angles = [math.pi * (c % 8) / 8 for c in range(C)]
