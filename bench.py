@@ -331,7 +331,9 @@ def main():
             torch.cuda.synchronize()
             m1 = time.perf_counter()
         gpu_ips = 128 * args.model_iters / (m1 - m0)
-        model_info = {"model": "ConvNeXt-T-1D inference, random init, bf16, batch 128, 3x224x224",
+        model_info = {"model": "ConvNeXt-T-1D inference, random init, bf16, batch 128, 3x224x224; "
+                               "oriented convs and the block/stem glue (LayerNorm, layout "
+                               "changes, residual) by this library, pointwise layers by PyTorch",
                       "images_per_s": round(gpu_ips, 1),
                       "ms_per_batch": round((m1 - m0) * 1e3 / args.model_iters, 2)}
         if not args.no_cpu_baseline:

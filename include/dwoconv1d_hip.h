@@ -106,6 +106,27 @@ int dwo_wgrad(const void *dy, const void *x, const void *taps, float *dw, float 
               int N, int C, int H, int W, int K, int stride, int dtype, int layout,
               void *stream);
 
+/*
+ * Forward-only glue of a ConvNeXt-1D block, each one pass over HBM in place of the PyTorch
+ * passes the reference spends around the operator (no counterpart in the reference's
+ * extension; they replace models/convnext.py:306-318 -- permute + LayerNorm before the
+ * pointwise layers, layer scale + permute + residual after them -- and the channels-last
+ * LayerNorm + GELU of the stem, :176-190).  LayerNorm is over the channel dimension, biased
+ * variance, fp32 statistics; gamma, beta and scale are fp32 [C]; C must be even.
+ *
+ * dwo_layernorm_nhwc:      out[r,:] = act(LN(x[r,:]) * gamma + beta) for rows of C contiguous
+ *                          channels (act = exact GELU when gelu != 0), C <= 2048.
+ * dwo_nchw_layernorm_nhwc: x [N,C,H,W] -> out [N,H,W,C] = LN over C * gamma + beta, C <= 1536.
+ * dwo_nhwc_scale_add_nchw: y [N,H,W,C] -> out [N,C,H,W] = res + scale[c] * y; scale and res
+ *                          (an [N,C,H,W] tensor) may be null, C <= 1536.
+ */
+int dwo_layernorm_nhwc(const void *x, const float *gamma, const float *beta, void *out,
+                       size_t rows, int C, float eps, int gelu, int dtype, void *stream);
+int dwo_nchw_layernorm_nhwc(const void *x, const float *gamma, const float *beta, void *out, int N,
+                            int C, int H, int W, float eps, int dtype, void *stream);
+int dwo_nhwc_scale_add_nchw(const void *y, const float *scale, const void *res, void *out, int N,
+                            int C, int H, int W, int dtype, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

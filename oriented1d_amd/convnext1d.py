@@ -15,6 +15,7 @@ import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
+from . import fused
 from .dwoconv1d import DepthwiseOrientedConv1d
 
 # (block kernel sizes, stem kernel size) per variant -- models/convnext.py:485-492
@@ -73,7 +74,11 @@ class ChannelsFirstLayerNorm(nn.Module):
         self.eps = eps
 
     def forward(self, x):
-        y = F.layer_norm(x.permute(0, 2, 3, 1), self.weight.shape, self.weight, self.bias, self.eps)
+        if fused.usable(x, x.shape[1], tiled=True):
+            y = fused.nchw_layernorm_nhwc(x, self.weight, self.bias, self.eps)
+        else:
+            y = F.layer_norm(x.permute(0, 2, 3, 1), self.weight.shape, self.weight, self.bias,
+                             self.eps)
         return y.permute(0, 3, 1, 2)
 
 
@@ -112,6 +117,15 @@ class Stem1D(nn.Module):
 
     def forward(self, x):
         x = self.pw1(x.permute(0, 2, 3, 1).contiguous())
+        if fused.usable(x, x.shape[-1], tiled=True) and fused.usable(x, self.pw2.out_features, True):
+            # the same values with each LayerNorm (+ GELU) and the final transpose as one pass
+            x = fused.layernorm_nhwc(self.dw1(x), self.norm1.weight, self.norm1.bias,
+                                     self.norm1.eps, gelu=True)
+            x = fused.layernorm_nhwc(self.dw2(x), self.norm2.weight, self.norm2.bias,
+                                     self.norm2.eps, gelu=True)
+            x = fused.layernorm_nhwc(self.pw2(x), self.norm3.weight, self.norm3.bias,
+                                     self.norm3.eps)
+            return fused.nhwc_scale_add_nchw(x)
         x = F.gelu(self.norm1(self.dw1(x)))
         x = F.gelu(self.norm2(self.dw2(x)))
         x = self.norm3(self.pw2(x))
@@ -144,11 +158,17 @@ class Block(nn.Module):
 
     def forward(self, x):
         y = (self.dwconv1 if self.plus_plus else self.dwconv)(x)
-        y = self.norm(y.permute(0, 2, 3, 1).contiguous())
+        fuse = fused.usable(y, y.shape[1], tiled=True) and not self.training
+        if fuse:  # permute + LayerNorm as one pass
+            y = fused.nchw_layernorm_nhwc(y, self.norm.weight, self.norm.bias, self.norm.eps)
+        else:
+            y = self.norm(y.permute(0, 2, 3, 1).contiguous())
         y = F.gelu(self.pwconv1(y))
         if self.plus_plus:
             y = self.dwconv2(y)
         y = self.pwconv2(y)
+        if fuse:  # layer scale + permute + residual as one pass (no stochastic depth in eval)
+            return fused.nhwc_scale_add_nchw(y, self.gamma, x)
         if self.gamma is not None:
             y = self.gamma * y
         return x + self.drop_path(y.permute(0, 3, 1, 2).contiguous())

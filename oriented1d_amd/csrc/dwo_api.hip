@@ -9,6 +9,7 @@
 #include "dwo_nhwc.h"
 #include "dwo_dispatch.h"
 #include "dwo_nhwc_tile.h"
+#include "dwo_fused.h"
 
 using namespace dwo;
 
@@ -415,6 +416,49 @@ int dwo_wgrad(const void *dy, const void *x, const void *taps, float *dw, float 
         case DWO_F32: return wgrad_t<float>(dy, x, taps, dw, db, scratch, d, layout, st);
         case DWO_BF16: return wgrad_t<bf16_t>(dy, x, taps, dw, db, scratch, d, layout, st);
         default: return wgrad_t<f16_t>(dy, x, taps, dw, db, scratch, d, layout, st);
+    }
+}
+
+int dwo_layernorm_nhwc(const void *x, const float *gamma, const float *beta, void *out,
+                       size_t rows, int C, float eps, int gelu, int dtype, void *stream) {
+    if (!x || !gamma || !beta || !out) return DWO_ERR_NULL_POINTER;
+    if (rows < 1 || C < 2 || (C & 1) || C > kFusedMaxC) return DWO_ERR_BAD_SHAPE;
+    hipStream_t st = (hipStream_t)stream;
+    switch (dtype) {
+        case DWO_F32: return launch_layernorm_nhwc<float>(x, gamma, beta, out, (long)rows, C, eps, gelu, st);
+        case DWO_BF16: return launch_layernorm_nhwc<bf16_t>(x, gamma, beta, out, (long)rows, C, eps, gelu, st);
+        case DWO_F16: return launch_layernorm_nhwc<f16_t>(x, gamma, beta, out, (long)rows, C, eps, gelu, st);
+        default: return DWO_ERR_BAD_DTYPE;
+    }
+}
+
+int dwo_nchw_layernorm_nhwc(const void *x, const float *gamma, const float *beta, void *out, int N,
+                            int C, int H, int W, float eps, int dtype, void *stream) {
+    if (!x || !gamma || !beta || !out) return DWO_ERR_NULL_POINTER;
+    if (N < 1 || N > 65535 || H < 1 || W < 1 || C < 2 || (C & 1) || C > kFusedMaxTileC ||
+        (long)H * W > 0x7fffffffL / C)
+        return DWO_ERR_BAD_SHAPE;
+    hipStream_t st = (hipStream_t)stream;
+    switch (dtype) {
+        case DWO_F32: return launch_nchw_layernorm_nhwc<float>(x, gamma, beta, out, N, C, H * W, eps, st);
+        case DWO_BF16: return launch_nchw_layernorm_nhwc<bf16_t>(x, gamma, beta, out, N, C, H * W, eps, st);
+        case DWO_F16: return launch_nchw_layernorm_nhwc<f16_t>(x, gamma, beta, out, N, C, H * W, eps, st);
+        default: return DWO_ERR_BAD_DTYPE;
+    }
+}
+
+int dwo_nhwc_scale_add_nchw(const void *y, const float *scale, const void *res, void *out, int N,
+                            int C, int H, int W, int dtype, void *stream) {
+    if (!y || !out) return DWO_ERR_NULL_POINTER;
+    if (N < 1 || N > 65535 || H < 1 || W < 1 || C < 2 || (C & 1) || C > kFusedMaxTileC ||
+        (long)H * W > 0x7fffffffL / C)
+        return DWO_ERR_BAD_SHAPE;
+    hipStream_t st = (hipStream_t)stream;
+    switch (dtype) {
+        case DWO_F32: return launch_nhwc_scale_add_nchw<float>(y, scale, res, out, N, C, H * W, st);
+        case DWO_BF16: return launch_nhwc_scale_add_nchw<bf16_t>(y, scale, res, out, N, C, H * W, st);
+        case DWO_F16: return launch_nhwc_scale_add_nchw<f16_t>(y, scale, res, out, N, C, H * W, st);
+        default: return DWO_ERR_BAD_DTYPE;
     }
 }
 
