@@ -118,7 +118,7 @@ int dwo_wgrad(const void *dy, const void *x, const void *taps, float *dw, float 
  *                          channels (act = exact GELU when gelu != 0), C <= 2048.
  * dwo_nchw_layernorm_nhwc: x [N,C,H,W] -> out [N,H,W,C] = LN over C * gamma + beta, C <= 1536.
  * dwo_nhwc_scale_add_nchw: y [N,H,W,C] -> out [N,C,H,W] = res + scale[c] * y; scale and res
- *                          (an [N,C,H,W] tensor) may be null, C <= 1536.
+ *                          (an [N,C,H,W] tensor) may be null.
  */
 int dwo_layernorm_nhwc(const void *x, const float *gamma, const float *beta, void *out,
                        size_t rows, int C, float eps, int gelu, int dtype, void *stream);

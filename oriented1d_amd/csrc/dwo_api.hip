@@ -450,8 +450,7 @@ int dwo_nchw_layernorm_nhwc(const void *x, const float *gamma, const float *beta
 int dwo_nhwc_scale_add_nchw(const void *y, const float *scale, const void *res, void *out, int N,
                             int C, int H, int W, int dtype, void *stream) {
     if (!y || !out) return DWO_ERR_NULL_POINTER;
-    if (N < 1 || N > 65535 || H < 1 || W < 1 || C < 2 || (C & 1) || C > kFusedMaxTileC ||
-        (long)H * W > 0x7fffffffL / C)
+    if (N < 1 || N > 65535 || H < 1 || W < 1 || C < 2 || (C & 1) || (long)H * W > 0x7fffffffL / C)
         return DWO_ERR_BAD_SHAPE;
     hipStream_t st = (hipStream_t)stream;
     switch (dtype) {

@@ -20,13 +20,16 @@ namespace dwo {
 
 constexpr int kFusedThreads = 256;
 constexpr int kFusedMaxC = 2048;          // 16 channel pairs per lane
-constexpr int kFusedMaxTileC = 1536;      // transposing kernels: 8 pixels x C floats within 64 KB
-constexpr int kFusedTileFloats = 12288;   // LDS tile of the transposing kernels (48 KB)
+constexpr int kFusedMaxTileC = 1536;      // transposing LayerNorm: 8 pixels x C floats within 64 KB
+constexpr int kFusedChanTile = 64;        // channels per workgroup of the transposing scale-add
 
-// pixels per tile for C channels: a power of two between 8 and 64 that fits the LDS tile
-inline int fused_tile_pixels(int C) {
+// Pixels per LDS tile [C][P + 1] of elements of `esize` bytes: the largest power of two up to 64
+// whose tile stays near 26 KB (six workgroups per CU), but not below 32 pixels -- shorter channel
+// rows waste most of every 128-byte line on the NCHW side -- while 32 still fit in 56 KB.
+inline int fused_tile_pixels(int C, int esize) {
     int p = 64;
-    while (p > 8 && (long)C * (p + 1) > kFusedTileFloats) p >>= 1;
+    while (p > 8 && (long)C * (p + 1) * esize > 26 * 1024) p >>= 1;
+    if (p < 32 && (long)C * 33 * esize <= 40 * 1024) p = 32;
     return p;
 }
 
@@ -107,6 +110,51 @@ __device__ __forceinline__ void normalise_and_store(float (&v)[2 * NP], int C, f
     }
 }
 
+// Sums over each half of a wave (lanes 0-31 and 32-63): the DPP reduction without its last
+// step; every lane gets its half's total.
+__device__ __forceinline__ float half_wave_total(float v) {
+#define DWO_DPP_ADD(ctrl, row_mask)                                                              \
+    v += __builtin_bit_cast(                                                                     \
+        float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), ctrl, row_mask, 0xf, true))
+    DWO_DPP_ADD(0x111, 0xf);  // row_shr:1
+    DWO_DPP_ADD(0x112, 0xf);  // row_shr:2
+    DWO_DPP_ADD(0x114, 0xf);  // row_shr:4
+    DWO_DPP_ADD(0x118, 0xf);  // row_shr:8
+    DWO_DPP_ADD(0x142, 0xa);  // row_bcast:15 into rows 1 and 3: lanes 31 and 63 hold the halves
+#undef DWO_DPP_ADD
+    const float lo = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 31));
+    const float hi = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
+    return (threadIdx.x & 32) ? hi : lo;
+}
+
+// Rows of at most 64 channels: two rows per wave, one per half, a lane holding one channel pair.
+template <typename T>
+__global__ __launch_bounds__(kFusedThreads) void layernorm_nhwc_narrow_kernel(
+    const T *__restrict__ x, const float *__restrict__ gamma, const float *__restrict__ beta,
+    T *__restrict__ out, long rows, int C, float eps, int gelu) {
+    const int c = 2 * (threadIdx.x & 31);
+    const bool live = c < C;
+    float g0 = 0.f, g1 = 0.f, b0 = 0.f, b1 = 0.f;
+    if (live) g0 = gamma[c], g1 = gamma[c + 1], b0 = beta[c], b1 = beta[c + 1];
+    const long first = ((long)blockIdx.x * (kFusedThreads / 64) + (threadIdx.x >> 6)) * 2 +
+                       ((threadIdx.x >> 5) & 1);
+    const long step = (long)gridDim.x * (kFusedThreads / 64) * 2;
+    const long last = (rows + 1) & ~1L;  // both halves of a wave run the same number of rounds
+    for (long r = first; r < last; r += step) {
+        float a = 0.f, b = 0.f;
+        const bool ok = live && r < rows;
+        if (ok) load_pair<T>(x + r * C + c, a, b);
+        const float mean = half_wave_total(a + b) / (float)C;
+        const float da = ok ? a - mean : 0.f, db = ok ? b - mean : 0.f;
+        const float rstd = rsqrtf(half_wave_total(da * da + db * db) / (float)C + eps);
+        if (ok) {
+            float u = da * rstd * g0 + b0, v = db * rstd * g1 + b1;
+            if (gelu) u = gelu_erf(u), v = gelu_erf(v);
+            store_pair<T>(out + r * C + c, u, v);
+        }
+    }
+}
+
 // rows of C contiguous channels; one wave per row, grid-stride over rows
 template <typename T, int NP>
 __global__ __launch_bounds__(kFusedThreads) void layernorm_nhwc_kernel(
@@ -127,59 +175,141 @@ __global__ __launch_bounds__(kFusedThreads) void layernorm_nhwc_kernel(
     }
 }
 
-// x [N,C,HW] -> out [N,HW,C], normalised over C.  Workgroup = (pixel tile, image).
-template <typename T, int NP>
-__global__ __launch_bounds__(kFusedThreads) void nchw_layernorm_nhwc_kernel(
-    const T *__restrict__ x, const float *__restrict__ gamma, const float *__restrict__ beta,
-    T *__restrict__ out, int C, int HW, int P, float eps) {
-    extern __shared__ float tile[];  // [C][P + 1]
-    const int n = blockIdx.y, p0 = blockIdx.x * P;
-    const int np = min(P, HW - p0);
-    const T *xn = x + (size_t)n * C * HW + p0;
-    // channel rows of P consecutive pixels: consecutive lanes read consecutive pixels
-    if (HW % 2 == 0) {  // (p0 and P are even: pairs of pixels stay aligned and inside the plane)
-        const int hp = P / 2;
-        for (int i = threadIdx.x; i < C * hp; i += kFusedThreads) {
-            const int c = i / hp, p = 2 * (i % hp);  // P is a power of two
-            if (p < np) {
-                float a, b;
-                load_pair<T>(xn + (size_t)c * HW + p, a, b);
-                tile[c * (P + 1) + p] = a;
-                tile[c * (P + 1) + p + 1] = b;
-            }
-        }
-    } else {
-        for (int i = threadIdx.x; i < C * P; i += kFusedThreads) {
-            const int c = i / P, p = i % P;
-            if (p < np) tile[c * (P + 1) + p] = to_float(xn[(size_t)c * HW + p]);
-        }
-    }
-    __syncthreads();
-    const int lane = threadIdx.x & 63;
-    T *on = out + ((size_t)n * HW + p0) * C;
-    for (int p = threadIdx.x >> 6; p < np; p += kFusedThreads / 64) {
-        float v[2 * NP];
+// NCHW side of the transposing kernels: channel rows of P consecutive pixels <-> the LDS tile
+// [C][P + 1].  With HW a multiple of four a lane moves four pixels (one 8- or 16-byte access);
+// all of a thread's loads are issued before their results are consumed.
+template <typename T, int VEC, class F>
+__device__ __forceinline__ void for_each_row_chunk(int C, int P, int np, F &&body) {
+    const int per_row = P / VEC;
+    const int total = C * per_row;
+    for (int i0 = threadIdx.x; i0 < total; i0 += 4 * kFusedThreads) {
 #pragma unroll
-        for (int k = 0; k < NP; k++) {
-            const int c = 2 * lane + 128 * k;
-            v[2 * k] = v[2 * k + 1] = 0.f;
-            if (c < C) v[2 * k] = tile[c * (P + 1) + p], v[2 * k + 1] = tile[(c + 1) * (P + 1) + p];
+        for (int u = 0; u < 4; u++) {
+            const int i = i0 + u * kFusedThreads;
+            const int c = i / per_row, p = VEC * (i % per_row);  // P is a power of two
+            body(u, i < total && p < np, c, p, false);
         }
-        normalise_and_store<T, NP>(v, C, eps, gamma, beta, false, on + (size_t)p * C);
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            const int i = i0 + u * kFusedThreads;
+            const int c = i / per_row, p = VEC * (i % per_row);
+            body(u, i < total && p < np, c, p, true);
+        }
     }
 }
 
-// y [N,HW,C] -> out [N,C,HW] = res + scale[c] * y (res and scale optional)
+template <typename T, int VEC>
+struct PixelVec;
 template <typename T>
-__global__ __launch_bounds__(kFusedThreads) void nhwc_scale_add_nchw_kernel(
-    const T *__restrict__ y, const float *__restrict__ scale, const T *__restrict__ res,
-    T *__restrict__ out, int C, int HW, int P) {
-    extern __shared__ float tile[];  // [C][P + 1]
+struct PixelVec<T, 4> : Vec4<T> {
+    __device__ __forceinline__ void load(const T *p) { this->load_cached(p); }
+    __device__ __forceinline__ void store(T *p) const { this->store_cached(p); }
+};
+template <typename T>
+struct PixelVec<T, 1> {
+    T v;
+    __device__ __forceinline__ void load(const T *p) { v = *p; }
+    __device__ __forceinline__ void store(T *p) const { *p = v; }
+    __device__ __forceinline__ float get(int) const { return to_float(v); }
+    __device__ __forceinline__ T elem(int) const { return v; }
+    __device__ __forceinline__ void set(float a, float, float, float) { v = from_float<T>(a); }
+};
+
+// x [N,C,HW] -> out [N,HW,C], normalised over C.  Workgroup = (pixel tile, image).  The
+// statistics of a pixel are gathered by kFusedThreads / P threads, each over a stride of the
+// channels (mean first, then the variance around it), and combined through LDS; then a wave
+// writes one pixel at a time, its lanes holding channel pairs.
+template <typename T, int NP, int VEC>
+__global__ __launch_bounds__(kFusedThreads) void nchw_layernorm_nhwc_kernel(
+    const T *__restrict__ x, const float *__restrict__ gamma, const float *__restrict__ beta,
+    T *__restrict__ out, int C, int HW, int P, float eps) {
+    // partial sums [G][P], mean [P], rstd [P], then the tile [C][P + 1] in the tensor's type
+    extern __shared__ float lds_fused[];
+    const int G = kFusedThreads / P;
+    float *part = lds_fused;
+    float *mean_s = part + G * P, *rstd_s = mean_s + P;
+    T *tile = reinterpret_cast<T *>(rstd_s + P);
     const int n = blockIdx.y, p0 = blockIdx.x * P;
     const int np = min(P, HW - p0);
-    const T *yn = y + ((size_t)n * HW + p0) * C;
-    // pixels of C contiguous channels, read as pairs
-    const int half = C / 2;
+    const T *xn = x + (size_t)n * C * HW + p0;
+    PixelVec<T, VEC> in[4];
+    for_each_row_chunk<T, VEC>(C, P, np, [&](int u, bool ok, int c, int p, bool second) {
+        if (!ok) return;
+        if (!second) {
+            in[u].load(xn + (size_t)c * HW + p);
+        } else {
+#pragma unroll
+            for (int e = 0; e < VEC; e++) tile[c * (P + 1) + p + e] = in[u].elem(e);
+        }
+    });
+    __syncthreads();
+    // statistics: thread (g, p) over channels g, g + G, ..
+    const int sp = threadIdx.x % P, sg = threadIdx.x / P;
+    float s = 0.f;
+    for (int c = sg; c < C; c += G) s += to_float(tile[c * (P + 1) + sp]);
+    part[sg * P + sp] = s;
+    __syncthreads();
+    float mean = 0.f;
+    for (int g = 0; g < G; g++) mean += part[g * P + sp];
+    mean /= (float)C;
+    float q = 0.f;
+    for (int c = sg; c < C; c += G) {
+        const float dlt = to_float(tile[c * (P + 1) + sp]) - mean;
+        q += dlt * dlt;
+    }
+    __syncthreads();  // every thread has read the partial sums
+    part[sg * P + sp] = q;
+    __syncthreads();
+    if (sg == 0) {
+        float var = 0.f;
+        for (int g = 0; g < G; g++) var += part[g * P + sp];
+        mean_s[sp] = mean;
+        rstd_s[sp] = rsqrtf(var / (float)C + eps);
+    }
+    __syncthreads();
+    const int lane = threadIdx.x & 63;
+    float gm[2 * NP], bt[2 * NP];
+#pragma unroll
+    for (int k = 0; k < NP; k++) {
+        const int c = 2 * lane + 128 * k;
+        gm[2 * k] = gm[2 * k + 1] = bt[2 * k] = bt[2 * k + 1] = 0.f;
+        if (c < C) gm[2 * k] = gamma[c], gm[2 * k + 1] = gamma[c + 1], bt[2 * k] = beta[c], bt[2 * k + 1] = beta[c + 1];
+    }
+    T *on = out + ((size_t)n * HW + p0) * C;
+    for (int p = threadIdx.x >> 6; p < np; p += kFusedThreads / 64) {
+        const float m = mean_s[p], r = rstd_s[p];
+#pragma unroll
+        for (int k = 0; k < NP; k++) {
+            const int c = 2 * lane + 128 * k;
+            if (c < C)
+                store_pair<T>(on + (size_t)p * C + c,
+                              (to_float(tile[c * (P + 1) + p]) - m) * r * gm[2 * k] + bt[2 * k],
+                              (to_float(tile[(c + 1) * (P + 1) + p]) - m) * r * gm[2 * k + 1] +
+                                  bt[2 * k + 1]);
+        }
+    }
+}
+
+// y [N,HW,C] -> out [N,C,HW] = res + scale[c] * y (res and scale optional).  Workgroup =
+// (pixel tile, channel tile, image): up to kFusedChanTile channels x P pixels.
+template <typename T, int VEC>
+__global__ __launch_bounds__(kFusedThreads) void nhwc_scale_add_nchw_kernel(
+    const T *__restrict__ y, const float *__restrict__ scale, const T *__restrict__ res,
+    T *__restrict__ out, int C, int HW, int P, int ptiles) {
+    extern __shared__ float tile[];  // [CT][P + 1]
+    const int n = blockIdx.y, p0 = (blockIdx.x % ptiles) * P, c0 = (blockIdx.x / ptiles) * kFusedChanTile;
+    const int np = min(P, HW - p0), CT = min(kFusedChanTile, C - c0);
+    const T *yn = y + ((size_t)n * HW + p0) * C + c0;
+    const size_t base = ((size_t)n * C + c0) * HW + p0;
+    // the residual rows do not depend on the tile: their loads go out first
+    PixelVec<T, VEC> rs[4];
+    const bool one_round = CT * (P / VEC) <= 4 * kFusedThreads;
+    if (res != nullptr && one_round)
+        for_each_row_chunk<T, VEC>(CT, P, np, [&](int u, bool ok, int c, int p, bool second) {
+            if (ok && !second) rs[u].load(res + base + (size_t)c * HW + p);
+        });
+    // pixels of CT contiguous channels, read as pairs
+    const int half = CT / 2;
     for (int i = threadIdx.x; i < half * np; i += kFusedThreads) {
         const int p = i / half, c = 2 * (i % half);
         float a, b;
@@ -188,33 +318,23 @@ __global__ __launch_bounds__(kFusedThreads) void nhwc_scale_add_nchw_kernel(
         tile[(c + 1) * (P + 1) + p] = b;
     }
     __syncthreads();
-    const size_t base = (size_t)n * C * HW + p0;
-    if (HW % 2 == 0) {  // two pixels per lane: 4-byte (8-byte fp32) accesses on the NCHW side
-        const int hp = P / 2;
-        for (int i = threadIdx.x; i < C * hp; i += kFusedThreads) {
-            const int c = i / hp, p = 2 * (i % hp);
-            if (p < np) {
-                float a = tile[c * (P + 1) + p], b = tile[c * (P + 1) + p + 1];
-                if (scale != nullptr) a *= scale[c], b *= scale[c];
-                if (res != nullptr) {
-                    float ra, rb;
-                    load_pair<T>(res + base + (size_t)c * HW + p, ra, rb);
-                    a += ra, b += rb;
-                }
-                store_pair<T>(out + base + (size_t)c * HW + p, a, b);
+    for_each_row_chunk<T, VEC>(CT, P, np, [&](int u, bool ok, int c, int p, bool second) {
+        if (!ok) return;
+        if (!second) {
+            if (res != nullptr && !one_round) rs[u].load(res + base + (size_t)c * HW + p);
+        } else {
+            float v[4] = {0.f, 0.f, 0.f, 0.f};
+            const float sc = scale != nullptr ? scale[c0 + c] : 1.f;
+#pragma unroll
+            for (int e = 0; e < VEC; e++) {
+                v[e] = tile[c * (P + 1) + p + e] * sc;
+                if (res != nullptr) v[e] += rs[u].get(e);
             }
+            PixelVec<T, VEC> o;
+            o.set(v[0], v[1], v[2], v[3]);
+            o.store(out + base + (size_t)c * HW + p);
         }
-    } else {
-        for (int i = threadIdx.x; i < C * P; i += kFusedThreads) {
-            const int c = i / P, p = i % P;
-            if (p < np) {
-                float v = tile[c * (P + 1) + p];
-                if (scale != nullptr) v *= scale[c];
-                if (res != nullptr) v += to_float(res[base + (size_t)c * HW + p]);
-                out[base + (size_t)c * HW + p] = from_float<T>(v);
-            }
-        }
-    }
+    });
 }
 
 // pairs per lane needed for C channels: 1, 2, 4, 8 or 16
@@ -238,6 +358,13 @@ int launch_layernorm_nhwc(const void *x, const float *gamma, const float *beta, 
                           int C, float eps, int gelu, hipStream_t st) {
     long blocks = (rows + kFusedThreads / 64 - 1) / (kFusedThreads / 64);
     if (blocks > 65536) blocks = 65536;
+    if (C <= 64) {
+        layernorm_nhwc_narrow_kernel<T><<<dim3((unsigned)((blocks + 1) / 2)), dim3(kFusedThreads), 0,
+                                          st>>>((const T *)x, gamma, beta, (T *)out, rows, C, eps,
+                                                gelu);
+        const hipError_t e = hipGetLastError();
+        return e == hipSuccess ? 0 : (int)e;
+    }
 #define DWO_CALL(NP_)                                                                        \
     layernorm_nhwc_kernel<T, NP_><<<dim3((unsigned)blocks), dim3(kFusedThreads), 0, st>>>(   \
         (const T *)x, gamma, beta, (T *)out, rows, C, eps, gelu)
@@ -250,12 +377,18 @@ int launch_layernorm_nhwc(const void *x, const float *gamma, const float *beta, 
 template <typename T>
 int launch_nchw_layernorm_nhwc(const void *x, const float *gamma, const float *beta, void *out,
                                int N, int C, int HW, float eps, hipStream_t st) {
-    const int P = fused_tile_pixels(C);
-    const size_t lds = (size_t)C * (P + 1) * sizeof(float);
+    const int P = fused_tile_pixels(C, (int)sizeof(T));
+    const size_t lds = ((size_t)kFusedThreads + 2 * P) * sizeof(float) + (size_t)C * (P + 1) * sizeof(T);
     const dim3 grid((HW + P - 1) / P, N), block(kFusedThreads);
-#define DWO_CALL(NP_)                                                    \
-    nchw_layernorm_nhwc_kernel<T, NP_><<<grid, block, lds, st>>>(        \
-        (const T *)x, gamma, beta, (T *)out, C, HW, P, eps)
+#define DWO_CALL(NP_)                                                              \
+    do {                                                                           \
+        if (HW % 4 == 0)                                                           \
+            nchw_layernorm_nhwc_kernel<T, NP_, 4><<<grid, block, lds, st>>>(       \
+                (const T *)x, gamma, beta, (T *)out, C, HW, P, eps);               \
+        else                                                                       \
+            nchw_layernorm_nhwc_kernel<T, NP_, 1><<<grid, block, lds, st>>>(       \
+                (const T *)x, gamma, beta, (T *)out, C, HW, P, eps);               \
+    } while (0)
     DWO_FUSED_NP_DISPATCH(C, DWO_CALL);
 #undef DWO_CALL
     const hipError_t e = hipGetLastError();
@@ -265,11 +398,16 @@ int launch_nchw_layernorm_nhwc(const void *x, const float *gamma, const float *b
 template <typename T>
 int launch_nhwc_scale_add_nchw(const void *y, const float *scale, const void *res, void *out, int N,
                                int C, int HW, hipStream_t st) {
-    const int P = fused_tile_pixels(C);
-    const size_t lds = (size_t)C * (P + 1) * sizeof(float);
-    const dim3 grid((HW + P - 1) / P, N), block(kFusedThreads);
-    nhwc_scale_add_nchw_kernel<T><<<grid, block, lds, st>>>((const T *)y, scale, (const T *)res,
-                                                           (T *)out, C, HW, P);
+    constexpr int P = 64;
+    const size_t lds = (size_t)kFusedChanTile * (P + 1) * sizeof(float);
+    const int ptiles = (HW + P - 1) / P, ctiles = (C + kFusedChanTile - 1) / kFusedChanTile;
+    const dim3 grid(ptiles * ctiles, N), block(kFusedThreads);
+    if (HW % 4 == 0)
+        nhwc_scale_add_nchw_kernel<T, 4><<<grid, block, lds, st>>>(
+            (const T *)y, scale, (const T *)res, (T *)out, C, HW, P, ptiles);
+    else
+        nhwc_scale_add_nchw_kernel<T, 1><<<grid, block, lds, st>>>(
+            (const T *)y, scale, (const T *)res, (T *)out, C, HW, P, ptiles);
     const hipError_t e = hipGetLastError();
     return e == hipSuccess ? 0 : (int)e;
 }
