@@ -107,6 +107,19 @@ int dwo_wgrad(const void *dy, const void *x, const void *taps, float *dw, float 
               void *stream);
 
 /*
+ * fprop of a pointwise-projected NHWC tensor without materialising it: y = fprop(pw(x)) with
+ * pw(x)[n,h,w,c] = pw_b[c] + sum_k x[n,h,w,k] * pw_w[c,k], rounded to the activation type as the
+ * separate layer's output would be.  The stem's first two layers of the reference
+ * (models/convnext.py:143,177-178: pw1 = nn.Linear(3, 64) then the stride-2 oriented
+ * convolution) in one pass: the 64-channel full-resolution tensor never goes to memory.
+ * x is [N,H,W,Cin] with Cin in {1,2,3,4}; pw_w [C,Cin] and pw_b [C] (may be null) are fp32; C must
+ * be a multiple of 4; the other arguments are those of dwo_fprop with layout DWO_NHWC.
+ */
+int dwo_pointwise_fprop_nhwc(const void *x, const float *pw_w, const float *pw_b, const float *w,
+                             const float *bias, const void *taps, void *y, int N, int Cin, int C,
+                             int H, int W, int K, int stride, int dtype, void *stream);
+
+/*
  * Forward-only glue of a ConvNeXt-1D block, each one pass over HBM in place of the PyTorch
  * passes the reference spends around the operator (no counterpart in the reference's
  * extension; they replace models/convnext.py:306-318 -- permute + LayerNorm before the

@@ -116,16 +116,22 @@ class Stem1D(nn.Module):
         self.norm3 = nn.LayerNorm(dim2, eps=1e-6)
 
     def forward(self, x):
-        x = self.pw1(x.permute(0, 2, 3, 1).contiguous())
-        if fused.usable(x, x.shape[-1], tiled=True) and fused.usable(x, self.pw2.out_features, True):
-            # the same values with each LayerNorm (+ GELU) and the final transpose as one pass
-            x = fused.layernorm_nhwc(self.dw1(x), self.norm1.weight, self.norm1.bias,
-                                     self.norm1.eps, gelu=True)
+        x = x.permute(0, 2, 3, 1).contiguous()
+        dw1 = self.dw1.conv if isinstance(self.dw1, ConvWrapper) else self.dw1
+        if (fused.usable(x, self.pw1.out_features, tiled=True) and x.shape[-1] <= 4
+                and self.pw1.out_features % 4 == 0
+                and fused.usable(x, self.pw2.out_features, tiled=True)):
+            # the same values with pw1 applied on the way into dw1 (its 64-channel output is
+            # never written), and each LayerNorm (+ GELU) and the final transpose as one pass
+            x = fused.pointwise_dwconv_nhwc(x, self.pw1, dw1)
+            x = fused.layernorm_nhwc(x, self.norm1.weight, self.norm1.bias, self.norm1.eps,
+                                     gelu=True)
             x = fused.layernorm_nhwc(self.dw2(x), self.norm2.weight, self.norm2.bias,
                                      self.norm2.eps, gelu=True)
             x = fused.layernorm_nhwc(self.pw2(x), self.norm3.weight, self.norm3.bias,
                                      self.norm3.eps)
             return fused.nhwc_scale_add_nchw(x)
+        x = self.pw1(x)
         x = F.gelu(self.norm1(self.dw1(x)))
         x = F.gelu(self.norm2(self.dw2(x)))
         x = self.norm3(self.pw2(x))

@@ -279,6 +279,18 @@ int wgrad_t(const void *dy, const void *x, const void *taps, float *dw, float *d
     return launch_status();
 }
 
+template <typename T>
+int pointwise_fprop_t(const void *x, const float *pw_w, const float *pw_b, const float *w,
+                      const float *bias, const void *taps, void *y, int Cin, const ConvDims &d,
+                      hipStream_t st) {
+    switch (Cin) {
+        case 1: return launch_nhwc_tile_pointwise_fprop<T, 1>(x, pw_w, pw_b, w, bias, taps, y, d, st);
+        case 2: return launch_nhwc_tile_pointwise_fprop<T, 2>(x, pw_w, pw_b, w, bias, taps, y, d, st);
+        case 3: return launch_nhwc_tile_pointwise_fprop<T, 3>(x, pw_w, pw_b, w, bias, taps, y, d, st);
+        default: return launch_nhwc_tile_pointwise_fprop<T, 4>(x, pw_w, pw_b, w, bias, taps, y, d, st);
+    }
+}
+
 }  // namespace
 
 extern "C" {
@@ -416,6 +428,22 @@ int dwo_wgrad(const void *dy, const void *x, const void *taps, float *dw, float 
         case DWO_F32: return wgrad_t<float>(dy, x, taps, dw, db, scratch, d, layout, st);
         case DWO_BF16: return wgrad_t<bf16_t>(dy, x, taps, dw, db, scratch, d, layout, st);
         default: return wgrad_t<f16_t>(dy, x, taps, dw, db, scratch, d, layout, st);
+    }
+}
+
+int dwo_pointwise_fprop_nhwc(const void *x, const float *pw_w, const float *pw_b, const float *w,
+                             const float *bias, const void *taps, void *y, int N, int Cin, int C,
+                             int H, int W, int K, int stride, int dtype, void *stream) {
+    int rc = check_common(N, C, H, W, K, stride, dtype, DWO_NHWC);
+    if (rc != DWO_OK) return rc;
+    if (!x || !pw_w || !w || !taps || !y) return DWO_ERR_NULL_POINTER;
+    if (Cin < 1 || Cin > 4 || C % kSliceCh != 0) return DWO_ERR_BAD_SHAPE;
+    const ConvDims d = make_dims(N, C, H, W, K, stride);
+    hipStream_t st = (hipStream_t)stream;
+    switch (dtype) {
+        case DWO_F32: return pointwise_fprop_t<float>(x, pw_w, pw_b, w, bias, taps, y, Cin, d, st);
+        case DWO_BF16: return pointwise_fprop_t<bf16_t>(x, pw_w, pw_b, w, bias, taps, y, Cin, d, st);
+        default: return pointwise_fprop_t<f16_t>(x, pw_w, pw_b, w, bias, taps, y, Cin, d, st);
     }
 }
 

@@ -67,16 +67,17 @@ __device__ __forceinline__ float from_float<float>(float v) {
 }
 template <>
 __device__ __forceinline__ bf16_t from_float<bf16_t>(float v) {
-    // round to nearest even; NaN stays NaN (quiet)
-    uint32_t u = __float_as_uint(v);
+    // round to nearest even in hardware (v_cvt_pk_bf16_f32)
     bf16_t r;
-    if ((u & 0x7fffffffu) > 0x7f800000u) {
-        r.bits = static_cast<uint16_t>((u >> 16) | 0x0040u);
-    } else {
-        u += 0x7fffu + ((u >> 16) & 1u);
-        r.bits = static_cast<uint16_t>(u >> 16);
-    }
+    r.bits = __builtin_bit_cast(uint16_t, (__bf16)v);
     return r;
+}
+// two values at once: (lo, hi) as one 32-bit word
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
+    typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
+    bf2 v;
+    v[0] = (__bf16)lo, v[1] = (__bf16)hi;
+    return __builtin_bit_cast(uint32_t, v);
 }
 template <>
 __device__ __forceinline__ f16_t from_float<f16_t>(float v) {

@@ -46,8 +46,7 @@ __device__ __forceinline__ void store_pair<float>(float *p, float a, float b) {
 }
 template <>
 __device__ __forceinline__ void store_pair<bf16_t>(bf16_t *p, float a, float b) {
-    *reinterpret_cast<uint32_t *>(p) =
-        (uint32_t)from_float<bf16_t>(a).bits | ((uint32_t)from_float<bf16_t>(b).bits << 16);
+    *reinterpret_cast<uint32_t *>(p) = pack_bf16(a, b);
 }
 template <>
 __device__ __forceinline__ void store_pair<f16_t>(f16_t *p, float a, float b) {

@@ -42,15 +42,90 @@ __device__ __forceinline__ void slice_load(Vec4<f16_t> &v, __amdgpu_buffer_rsrc_
     v.v = __builtin_bit_cast(Vec4<f16_t>::h4, __builtin_amdgcn_raw_buffer_load_b64(r, off, 0, 0));
 }
 
+// Where the window's pixels come from.  SliceSource: an NHWC tensor with the convolution's own
+// channel count; a pixel's payload is the workgroup's four-channel slice.  PointwiseSource: an
+// NHWC tensor of CIN channels (the network's input image) to which a pointwise linear layer
+// CIN -> C is applied on the way into LDS (the stem's first layer, models/convnext.py:143,177:
+// the C-channel tensor is never written to memory); out-of-image positions are zeros of the
+// *projected* tensor, and the projection is rounded to the activation type as the separate layer's
+// output would be.
+template <typename T>
+struct SliceSource {
+    typedef Vec4<T> Payload;
+    struct Params {
+        const T *x;
+    };
+    __amdgpu_buffer_rsrc_t img;
+    unsigned pix_bytes;
+    __device__ __forceinline__ void init(const Params &p, int n, int c0, const ConvDims &d) {
+        const T *xn = p.x + (size_t)n * d.H * d.W * d.C + c0;
+        img = __builtin_amdgcn_make_buffer_rsrc(
+            const_cast<T *>(xn), 0, (unsigned)(((size_t)d.H * d.W * d.C - c0) * sizeof(T)), 0x00020000);
+        pix_bytes = d.C * (unsigned)sizeof(T);
+    }
+    // (positions outside the image get an offset beyond the descriptor and read as zeros, so the
+    // loads need no predicates)
+    __device__ __forceinline__ void load(Payload &v, bool inside, unsigned pixel) const {
+        slice_load(v, img, inside ? pixel * pix_bytes : 0xffffffffu);
+    }
+    __device__ __forceinline__ T elem(const Payload &v, int ch, bool) const { return v.elem(ch); }
+};
+
+__device__ __forceinline__ float buffer_value(__amdgpu_buffer_rsrc_t r, unsigned off, float) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, off, 0, 0));
+}
+__device__ __forceinline__ float buffer_value(__amdgpu_buffer_rsrc_t r, unsigned off, bf16_t) {
+    return __uint_as_float((unsigned)__builtin_amdgcn_raw_buffer_load_b16(r, off, 0, 0) << 16);
+}
+__device__ __forceinline__ float buffer_value(__amdgpu_buffer_rsrc_t r, unsigned off, f16_t) {
+    return (float)__builtin_bit_cast(_Float16, __builtin_amdgcn_raw_buffer_load_b16(r, off, 0, 0));
+}
+
+template <typename T, int CIN>
+struct PointwiseSource {
+    struct Payload {
+        float v[CIN];
+    };
+    struct Params {
+        const T *x;         // [N,H,W,CIN]
+        const float *pw_w;  // [C,CIN]
+        const float *pw_b;  // [C] or null
+    };
+    __amdgpu_buffer_rsrc_t img;
+    float w[kSliceCh][CIN], b[kSliceCh];
+    __device__ __forceinline__ void init(const Params &p, int n, int c0, const ConvDims &d) {
+        const T *xn = p.x + (size_t)n * d.H * d.W * CIN;
+        img = __builtin_amdgcn_make_buffer_rsrc(
+            const_cast<T *>(xn), 0, (unsigned)((size_t)d.H * d.W * CIN * sizeof(T)), 0x00020000);
+#pragma unroll
+        for (int ch = 0; ch < kSliceCh; ch++) {
+            b[ch] = p.pw_b != nullptr ? p.pw_b[c0 + ch] : 0.f;
+#pragma unroll
+            for (int k = 0; k < CIN; k++) w[ch][k] = p.pw_w[(size_t)(c0 + ch) * CIN + k];
+        }
+    }
+    __device__ __forceinline__ void load(Payload &v, bool inside, unsigned pixel) const {
+#pragma unroll
+        for (int k = 0; k < CIN; k++)
+            v.v[k] = buffer_value(img, inside ? (pixel * CIN + k) * (unsigned)sizeof(T) : 0xffffffffu, T{});
+    }
+    __device__ __forceinline__ T elem(const Payload &v, int ch, bool inside) const {
+        float a = b[ch];
+#pragma unroll
+        for (int k = 0; k < CIN; k++) a = __builtin_fmaf(v.v[k], w[ch][k], a);
+        return inside ? from_float<T>(a) : T{};
+    }
+};
+
 // floor(n / d) for n < 2^16 and 2 <= d < 2^16, with m = ceil(2^32 / d)
 __device__ __forceinline__ unsigned fast_div(unsigned n, unsigned m) { return __umulhi(n, m); }
 __device__ __forceinline__ unsigned div_magic(unsigned d) {
     return (unsigned)((0x100000000ull + d - 1) / d);
 }
 
-template <typename T>
+template <typename T, class Src>
 __global__ __launch_bounds__(kTileThreads) __attribute__((amdgpu_waves_per_eu(4, 4))) void nhwc_tile_fprop_kernel(
-    const T *__restrict__ x, const float *__restrict__ wt, const float *__restrict__ bias,
+    typename Src::Params sp, const float *__restrict__ wt, const float *__restrict__ bias,
     const int8_t *__restrict__ dhdw, T *__restrict__ y, ConvDims d, int nbands, int tasks_per_image) {
     extern __shared__ float lds_f[];
     T *planes = reinterpret_cast<T *>(lds_f);
@@ -123,29 +198,31 @@ __global__ __launch_bounds__(kTileThreads) __attribute__((amdgpu_waves_per_eu(4,
         mytab[stid] = make_int2(((int)mytaps[2 * stid] / rstep) * iwp + (int)mytaps[2 * stid + 1] / cstep,
                                 __float_as_int(wt[(size_t)c * K + stid]));
 
-    const T *xn = x + (size_t)n * d.H * d.W * d.C + c0;
     T *yn = y + (size_t)n * d.P * d.Q * d.C + c0;
     const T *plane = planes + sub * kTilePlaneElems;
     const unsigned nwin = ih * iw, nout = th * tw;
 
     // window of sub-tile (pt, qt) -> registers: rows pt*s - hh .., columns qt*s - hw ..
-    // (through a buffer descriptor over the image: positions outside it get an offset beyond
-    // the descriptor and read as zeros, so the loads need no predicates)
-    constexpr int PRE = kTilePlaneElems / kTileThreads;  // slices per thread, at most
-    Vec4<T> pre[PRE];
-    const __amdgpu_buffer_rsrc_t img = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<T *>(xn), 0, (unsigned)(((size_t)d.H * d.W * d.C - c0) * sizeof(T)), 0x00020000);
+    constexpr int PRE = kTilePlaneElems / kTileThreads;  // pixels per thread, at most
+    typename Src::Payload pre[PRE];
+    Src source;
+    source.init(sp, n, c0, d);
+    auto window_pixel = [&](int pt, int qt, unsigned v, unsigned &pixel) {
+        const unsigned i = fast_div(v, m_iw), j = v - i * iw;
+        const unsigned r = (unsigned)(pt * s_ - hh + (int)i * rstep);
+        const unsigned q = (unsigned)(qt * s_ - hw + (int)j * cstep);
+        pixel = r * d.W + q;
+        return v < nwin && r < (unsigned)d.H && q < (unsigned)d.W;
+    };
     auto load_window = [&](int pt, int qt) {
-        const int r0 = pt * s_ - hh, q0 = qt * s_ - hw;
 #pragma unroll
         for (int u = 0; u < PRE; u++) {
             if (u * kTileThreads >= (int)nwin) break;
             unsigned v = u * kTileThreads + threadIdx.x;
             asm volatile("" : "+v"(v));  // recompute per window: hoisting 16 index sets spills
-            const unsigned i = fast_div(v, m_iw), j = v - i * iw;
-            const unsigned r = (unsigned)(r0 + (int)i * rstep), q = (unsigned)(q0 + (int)j * cstep);
-            const bool inside = v < nwin && r < (unsigned)d.H && q < (unsigned)d.W;
-            slice_load(pre[u], img, inside ? (r * d.W + q) * d.C * (unsigned)sizeof(T) : 0xffffffffu);
+            unsigned pixel;
+            const bool inside = window_pixel(pt, qt, v, pixel);
+            source.load(pre[u], inside, pixel);
         }
     };
     load_window(p_lo, 0);
@@ -159,9 +236,11 @@ __global__ __launch_bounds__(kTileThreads) __attribute__((amdgpu_waves_per_eu(4,
                 if (v < nwin) {
                     const unsigned i = fast_div(v, m_iw), j = v - i * iw;
                     const unsigned at = i * iwp + j;
+                    unsigned pixel;
+                    const bool inside = window_pixel(pt, qt, v, pixel);
 #pragma unroll
                     for (int ch = 0; ch < kSliceCh; ch++)
-                        planes[ch * kTilePlaneElems + at] = pre[u].elem(ch);
+                        planes[ch * kTilePlaneElems + at] = source.elem(pre[u], ch, inside);
                 }
             }
             __syncthreads();
@@ -210,12 +289,12 @@ __global__ __launch_bounds__(kTileThreads) __attribute__((amdgpu_waves_per_eu(4,
 }
 
 // grid: 8 * ceil(N / 8) * bands * slices workgroups
-template <typename T>
-int launch_nhwc_tile_fprop(const void *x, const float *w, const float *bias, const void *taps,
-                           void *y, const ConvDims &d, hipStream_t st) {
+template <typename T, class Src>
+int launch_nhwc_tile(const typename Src::Params &sp, const float *w, const float *bias,
+                     const void *taps, void *y, const ConvDims &d, hipStream_t st) {
     const size_t lds = nhwc_tile_lds_bytes<T>();
     static const bool once = [&] {
-        allow_large_lds(nhwc_tile_fprop_kernel<T>, lds);
+        allow_large_lds(nhwc_tile_fprop_kernel<T, Src>, lds);
         return true;
     }();
     (void)once;
@@ -223,10 +302,25 @@ int launch_nhwc_tile_fprop(const void *x, const float *w, const float *bias, con
     const int tpi = nbands * (d.C / kSliceCh);
     const long grid = 8L * ((d.N + 7) / 8) * tpi;
     if (grid > 0x7fffffffL) return DWO_ERR_BAD_SHAPE;
-    nhwc_tile_fprop_kernel<T><<<dim3((unsigned)grid), dim3(kTileThreads), lds, st>>>(
-        (const T *)x, w, bias, taps_dhdw(taps), (T *)y, d, nbands, tpi);
+    nhwc_tile_fprop_kernel<T, Src><<<dim3((unsigned)grid), dim3(kTileThreads), lds, st>>>(
+        sp, w, bias, taps_dhdw(taps), (T *)y, d, nbands, tpi);
     const hipError_t e = hipGetLastError();
     return e == hipSuccess ? 0 : (int)e;
+}
+
+template <typename T>
+int launch_nhwc_tile_fprop(const void *x, const float *w, const float *bias, const void *taps,
+                           void *y, const ConvDims &d, hipStream_t st) {
+    return launch_nhwc_tile<T, SliceSource<T>>({(const T *)x}, w, bias, taps, y, d, st);
+}
+
+// fprop of the C-channel tensor pw(x): x [N,H,W,CIN], pw_w [C,CIN], pw_b [C] or null
+template <typename T, int CIN>
+int launch_nhwc_tile_pointwise_fprop(const void *x, const float *pw_w, const float *pw_b,
+                                     const float *w, const float *bias, const void *taps, void *y,
+                                     const ConvDims &d, hipStream_t st) {
+    return launch_nhwc_tile<T, PointwiseSource<T, CIN>>({(const T *)x, pw_w, pw_b}, w, bias, taps, y,
+                                                         d, st);
 }
 
 }  // namespace dwo

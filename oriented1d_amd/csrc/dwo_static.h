@@ -80,8 +80,8 @@ struct Vec4<bf16_t> {
     __device__ __forceinline__ bf16_t elem(int i) const { return bf16_t{bits(i)}; }
     __device__ __forceinline__ void clear() { v = u2{0u, 0u}; }
     __device__ __forceinline__ void set(float a, float b, float c, float d) {
-        v.x = (uint32_t)from_float<bf16_t>(a).bits | ((uint32_t)from_float<bf16_t>(b).bits << 16);
-        v.y = (uint32_t)from_float<bf16_t>(c).bits | ((uint32_t)from_float<bf16_t>(d).bits << 16);
+        v.x = pack_bf16(a, b);
+        v.y = pack_bf16(c, d);
     }
 };
 template <>

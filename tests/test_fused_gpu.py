@@ -70,6 +70,36 @@ def test_nhwc_scale_add_nchw(N, C, H, W, with_scale, with_res, dtype):
     _close(got, ref, dtype, "nhwc_scale_add_nchw")
 
 
+@pytest.mark.parametrize("dtype", DTYPES, ids=["f32", "bf16", "f16"])
+@pytest.mark.parametrize("Cin,C,H,W,K,stride", [(3, 64, 64, 48, 31, 2), (3, 24, 37, 29, 15, 2),
+                                               (4, 8, 20, 20, 7, 1), (1, 16, 33, 70, 31, 4)])
+def test_pointwise_then_oriented_conv(oracle, Cin, C, H, W, K, stride, dtype):
+    """dwo_pointwise_fprop_nhwc against the two separate layers: nn.Linear Cin -> C rounded to
+    the activation type (what the reference's pw1 hands to dw1, models/convnext.py:177-178),
+    then the oracle's fprop with bias."""
+    import numpy as np
+    from parity_util import grouped_theta, rounded
+    from oriented1d_amd.dwoconv1d import DepthwiseOrientedConv1d
+
+    torch.manual_seed(Cin * 100 + C)
+    lin = torch.nn.Linear(Cin, C).cuda()
+    conv = DepthwiseOrientedConv1d(C, C, K, groups=C, stride=stride, padding=K // 2, bias=True,
+                                   angle=grouped_theta(C).tolist(), nhwc=True).cuda()
+    torch.nn.init.normal_(conv.bias, std=0.3)
+    x = torch.randn(2, H, W, Cin, device="cuda").to(dtype)
+    with torch.no_grad():
+        got = fused.pointwise_dwconv_nhwc(x, lin, conv)
+    mid = x.double().cpu().numpy() @ lin.weight.detach().double().cpu().numpy().T \
+        + lin.bias.detach().double().cpu().numpy()
+    mid = rounded(mid.astype(np.float32), dtype)  # the separate layer's output in the tensor's type
+    ref = oracle.fprop(np.ascontiguousarray(mid.transpose(0, 3, 1, 2)),
+                       conv.weight.detach().cpu().numpy(), conv.theta.detach().cpu().numpy(), stride)
+    ref = ref + conv.bias.detach().double().cpu().numpy().reshape(1, -1, 1, 1)
+    P, Q = -(-H // stride), -(-W // stride)
+    assert got.shape == (2, P, Q, C) and got.dtype == dtype
+    _close(got.permute(0, 3, 1, 2), torch.from_numpy(ref), dtype, "pointwise_fprop")
+
+
 def test_argument_errors():
     x = torch.randn(2, 7, 4, 4, device="cuda")  # odd channel count
     with pytest.raises(RuntimeError):
