@@ -304,6 +304,17 @@ class DepthwiseOrientedConv1d(nn.Conv2d):
             self.resid = None
         self._taps = _TapCache()
 
+    def _apply(self, fn, recurse=True):
+        """``.to()/.half()/.bfloat16()/.cuda()`` move and cast weight and bias, but the angles stay
+        fp32: they are geometry, and their tap offsets (``(int)(cosf(theta) * k)``) change when
+        theta is rounded to a 16-bit type (the reference supports fp32 only and would
+        reinterpret the bits, kernels.cu:25)."""
+        theta = self.theta.data
+        super()._apply(fn, recurse)
+        if self.theta.dtype != torch.float32:
+            self.theta.data = theta.to(self.theta.device)
+        return self
+
     def forward_safe(self, x):
         """Arbitrary H, W (reference: dwoconv1d.py:154-187); handled natively."""
         return self.forward(x)

@@ -137,3 +137,22 @@ def test_oracle_reproduces_golden_fixture(oracle):
     np.testing.assert_array_equal(y, g["y"])
     dw = oracle.wgrad(dy, x, theta, 31, threads=4).reshape(96, 31)
     np.testing.assert_array_equal(dw, g["dw"])
+
+
+def test_angles_stay_fp32_under_module_casts():
+    """Casting the module to a 16-bit type must not round theta: the tap offsets of the rounded
+    angles differ from those of the fp32 ones."""
+    C, K = 16, 31
+    angles = [math.pi * (c % 8) / 8 for c in range(C)]
+    m = op.DepthwiseOrientedConv1d(C, C, K, groups=C, padding=K // 2, angle=angles)
+    before = m.theta.detach().clone()
+    for cast in (lambda mod: mod.bfloat16(), lambda mod: mod.half(), lambda mod: mod.to(torch.float64),
+                 lambda mod: mod.float()):
+        m = cast(m)
+        assert m.theta.dtype == torch.float32 and torch.equal(m.theta.detach(), before)
+    assert m.weight.dtype == torch.float32
+    assert m.bfloat16().weight.dtype == torch.bfloat16
+    rounded_theta = before.to(torch.bfloat16).float()
+    dh0, dw0 = op.taps_to_numpy(op.build_taps(before, C, K), C, K)
+    dh1, dw1 = op.taps_to_numpy(op.build_taps(rounded_theta, C, K), C, K)
+    assert (dh0 != dh1).any() or (dw0 != dw1).any()
