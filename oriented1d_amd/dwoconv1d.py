@@ -18,6 +18,7 @@ Differences from the reference, all supersets:
   ceil(H/stride) x ceil(W/stride) outputs, the same values that path produces.
 """
 import ctypes
+import weakref
 
 import numpy as np
 import torch
@@ -110,6 +111,25 @@ def _w2d(w, C):
     return w.to(torch.float32).contiguous()
 
 
+_F32_COPIES = {}  # id(parameter) -> (weak reference, state key, fp32 copy)
+
+
+def f32_copy(p):
+    """fp32 contiguous copy of a parameter, kept until the parameter is modified or moved (the
+    library takes weights, biases and norm parameters as fp32; re-casting 16-bit parameters at
+    every call costs a kernel launch each)."""
+    if p.dtype == torch.float32 and p.is_contiguous():
+        return p.detach()
+    key = (p._version, p.data_ptr(), p.dtype, str(p.device))
+    hit = _F32_COPIES.get(id(p))
+    if hit is None or hit[0]() is not p or hit[1] != key:
+        pid = id(p)
+        ref = weakref.ref(p, lambda _, pid=pid: _F32_COPIES.pop(pid, None))
+        hit = (ref, key, p.detach().to(torch.float32).contiguous())
+        _F32_COPIES[pid] = hit
+    return hit[2]
+
+
 def fprop(x, w, taps, stride=1, bias=None, nhwc=False):
     """y = fprop(x, w, theta) (+ bias).  x: [N,C,H,W] or [N,H,W,C]; w: [C,1,1,K]."""
     lib = _lib.load()
@@ -117,7 +137,7 @@ def fprop(x, w, taps, stride=1, bias=None, nhwc=False):
     N, C, H, W = _dims(x, nhwc)
     w2 = _w2d(w, C)
     K = w2.shape[1]
-    b = bias.detach().to(torch.float32).contiguous() if bias is not None else None
+    b = f32_copy(bias) if bias is not None else None
     y = torch.empty(_out_shape(N, C, H, W, stride, nhwc), dtype=x.dtype, device=x.device)
     _lib.check(lib.dwo_fprop(_ptr(x), _ptr(w2), _ptr(b), _ptr(taps), _ptr(y), N, C, H, W, K,
                              stride, _DTYPES[x.dtype], int(nhwc), _stream(x)), "dwo_fprop")
@@ -173,7 +193,7 @@ class _DepthwiseOrientedConv1d(torch.autograd.Function):
         stride = module.stride[0]
         C = w.shape[0]
         K = w.shape[-1]
-        w_eff = w.detach().to(torch.float32)
+        w_eff = f32_copy(w)
         if resid is not None:
             w_eff = w_eff + resid.to(w_eff)
         x = x.contiguous()

@@ -22,7 +22,8 @@ def _stream(t):
 
 
 def _f32(p):
-    return p.detach().to(torch.float32).contiguous()
+    from .dwoconv1d import f32_copy
+    return f32_copy(p)
 
 
 def usable(x, C, tiled):
@@ -89,15 +90,15 @@ def pointwise_dwconv_nhwc(x, linear, conv):
     x = x.contiguous()
     N, H, W, Cin = x.shape
     C, K, stride = conv.out_channels, conv.kernel_size[1], conv.stride[0]
-    w = conv.weight.detach()
+    w = _f32(conv.weight)
     if conv.resid is not None:
-        w = w + conv.resid
+        w = w + conv.resid.to(w)
     taps = conv._taps.get(conv.theta, C, K, x.device)  # cached per theta version
     P, Q = -(-H // stride), -(-W // stride)
     y = torch.empty((N, P, Q, C), dtype=x.dtype, device=x.device)
     pw_w = _f32(linear.weight)
     pw_b = _f32(linear.bias) if linear.bias is not None else None
-    w2 = _f32(w).reshape(C, K)
+    w2 = w.reshape(C, K)
     cb = _f32(conv.bias) if conv.bias is not None else None
     _lib.check(_lib.load().dwo_pointwise_fprop_nhwc(
         _ptr(x), _ptr(pw_w), _ptr(pw_b), _ptr(w2), _ptr(cb), _ptr(taps), _ptr(y), N, Cin, C, H, W,

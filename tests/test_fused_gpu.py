@@ -129,3 +129,24 @@ def test_block_and_stem_fused_equal_unfused(variant):
         y_fused = m(x)
     y_plain = m(x.requires_grad_(True))  # gradient recording switches the glue kernels off
     _close(y_fused, y_plain.detach(), torch.float32, "network")
+
+
+def test_bf16_network_fused_equal_unfused_and_parameter_copies_refresh():
+    """The 16-bit network (parameters cast with .bfloat16(): the library works from cached fp32
+    copies of them) with and without the glue kernels, and the copies follow in-place updates."""
+    from oriented1d_amd.convnext1d import ConvNeXt1D
+
+    torch.manual_seed(4)
+    m = ConvNeXt1D(depths=(1, 1, 1, 1), dims=(16, 32, 64, 128), variant="1d", stem_dim1=24,
+                   num_classes=10, layer_scale_init_value=1.0).cuda().bfloat16().eval()
+    x = torch.randn(2, 3, 64, 64, device="cuda").bfloat16()
+    with torch.no_grad():
+        y_fused = m(x)
+    y_plain = m(x.requires_grad_(True)).detach()
+    _close(y_fused, y_plain, torch.bfloat16, "bf16 network")
+    with torch.no_grad():
+        m.stages[0][0].dwconv.weight.mul_(3.0)   # in-place update: the cached copy must refresh
+        y_fused2 = m(x.detach())
+    y_plain2 = m(x).detach()
+    _close(y_fused2, y_plain2, torch.bfloat16, "bf16 network after update")
+    assert not torch.equal(y_fused, y_fused2)
