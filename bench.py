@@ -60,6 +60,9 @@ def main():
     ap.add_argument("--only", default="", help="restrict the per-kernel table, e.g. 96x56:fprop")
     ap.add_argument("--model-iters", type=int, default=5,
                     help="timed ConvNeXt-T-1D inference forwards (batch 128, bf16); 0 skips it")
+    ap.add_argument("--train-iters", type=int, default=3,
+                    help="timed steps of the two training configurations (ConvNeXt-B-1D++ "
+                         "training, ConvNeXt-T-1D features fwd+bwd); 0 skips them")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="also run a plain device copy of one 96x56x56 batch-64 tensor (a kernel "
                          "of known traffic, for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE)")
@@ -370,6 +373,73 @@ def main():
                                         "CPU ops with %d threads, oriented convs by the oracle's "
                                         "loops on %d threads" % (torch.get_num_threads(), nthreads))
 
+    # ------------------------------------------------------------------ the two training configurations
+    # ConvNeXt-B-1D++ training step (fwd + bwd + AdamW, bf16 autocast over fp32 masters, batch 64,
+    # stochastic depth 0.5, random labels) and ConvNeXt-T-1D dense features at 8 x 3 x 512 x 512
+    # (bf16, the four stage outputs, loss = sum <out_i, R_i>, fwd + bwd).  Reported, not part of
+    # `value`.
+    train_info = None
+    if args.train_iters > 0:
+        model = None
+        torch.cuda.empty_cache()
+        from oriented1d_amd.convnext1d import convnext_base_1d, convnext_tiny_1d
+        train_info = {}
+        try:
+            torch.manual_seed(0)
+            net = convnext_base_1d(variant="1dpp", drop_path_rate=0.5).to(dev).train()
+            opt = torch.optim.AdamW(net.parameters(), lr=1e-3, weight_decay=0.05)
+            imgs = torch.randn(64, 3, 224, 224, device=dev)
+            labels = torch.randint(0, 1000, (64,), device=dev)
+
+            def train_step():
+                opt.zero_grad(set_to_none=True)
+                with torch.autocast("cuda", dtype=torch.bfloat16):
+                    loss = torch.nn.functional.cross_entropy(net(imgs).float(), labels)
+                loss.backward()
+                opt.step()
+
+            for _ in range(2):
+                train_step()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(args.train_iters):
+                train_step()
+            torch.cuda.synchronize()
+            dt = (time.perf_counter() - t0) / args.train_iters
+            train_info["convnext_b_1dpp_train"] = {
+                "config": "fwd+bwd+AdamW, bf16 autocast, batch 64, 3x224x224, drop path 0.5",
+                "ms_per_step": round(dt * 1e3, 2), "images_per_s": round(64 / dt, 1)}
+            del net, opt, imgs, labels
+            torch.cuda.empty_cache()
+
+            net = convnext_tiny_1d(variant="1d", out_stages=True).to(dev).to(torch.bfloat16).train()
+            imgs = torch.randn(8, 3, 512, 512, device=dev).to(torch.bfloat16)
+            targets = []
+
+            def feature_step():
+                for p_ in net.parameters():
+                    p_.grad = None
+                outs = net(imgs)
+                if not targets:
+                    targets.extend(torch.randn_like(o) for o in outs)
+                sum((o.float() * r.float()).sum() for o, r in zip(outs, targets)).backward()
+
+            for _ in range(2):
+                feature_step()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(args.train_iters):
+                feature_step()
+            torch.cuda.synchronize()
+            dt = (time.perf_counter() - t0) / args.train_iters
+            train_info["convnext_t_1d_features"] = {
+                "config": "fwd+bwd, bf16, 8x3x512x512, four stage outputs, loss = sum <out_i, R_i>",
+                "ms_per_step": round(dt * 1e3, 2), "images_per_s": round(8 / dt, 1)}
+            del net, imgs, targets
+        except RuntimeError as exc:  # e.g. out of memory next to another process: keep the main line
+            train_info["error"] = str(exc).splitlines()[0][:200]
+        torch.cuda.empty_cache()
+
     out = {
         "metric": "dwoconv1d fprop/dgrad/wgrad GB/s (% HBM peak); ConvNeXt-T-1D img/s",
         "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
@@ -386,7 +456,7 @@ def main():
         "frac_hbm_peak": round(value / HBM_PEAK_GBS, 4),
         "detail": detail, "roofline": roofline, "cpu_baseline": cpu,
         "cpu_baseline_all_threads": cpu_all, "other_configs": others,
-        "convnext_t_1d": model_info,
+        "convnext_t_1d": model_info, "training_configs": train_info,
     }
     print(json.dumps(out))
 
