@@ -157,13 +157,16 @@ int wgrad_max_partials(const ConvDims &d, int layout) {
     return nbatch < kMaxPlaneGroups ? nbatch : kMaxPlaneGroups;
 }
 
-// NHWC fprop at any extent and stride with the channel count a multiple of 4: slice tiles
+// fprop (flip = 0) or stride-1 dgrad (flip = 1) at any extent by the tile kernel: NCHW always,
+// NHWC with the channel count a multiple of 4; images up to 4 GB (32-bit offsets inside one)
 template <typename T>
-int try_nhwc_tile_fprop(const void *x, const float *w, const float *bias, const void *taps, void *y,
-                        const ConvDims &d, int layout, hipStream_t st) {
-    if (layout != DWO_NHWC || d.C % kSliceCh != 0) return -100;
-    if ((size_t)d.H * d.W * d.C * sizeof(T) >= 0xffffffffull) return -100;  // 32-bit image offsets
-    return launch_nhwc_tile_fprop<T>(x, w, bias, taps, y, d, st);
+int try_tile_conv(const void *x, const float *w, const float *bias, const void *taps, void *y,
+                  const ConvDims &d, int layout, int flip, hipStream_t st) {
+    if (flip && d.stride != 1) return -100;
+    if ((size_t)d.H * d.W * d.C * sizeof(T) >= 0xffffffffull) return -100;
+    if (layout == DWO_NCHW) return launch_nchw_tile_fprop<T>(x, w, bias, taps, y, d, flip, st);
+    if (d.C % kSliceCh != 0) return -100;
+    return launch_nhwc_tile_fprop<T>(x, w, bias, taps, y, d, flip, st);
 }
 
 template <typename T, int MODE>
@@ -208,7 +211,7 @@ int fprop_t(const void *x, const float *w, const float *bias, const void *taps, 
     if (fast != -100) return fast;
     const int sliced = try_nhwc_plane_conv<T>(OP_FPROP, x, w, bias, taps, y, d, layout, st);
     if (sliced != -100) return sliced;
-    const int tiled = try_nhwc_tile_fprop<T>(x, w, bias, taps, y, d, layout, st);
+    const int tiled = try_tile_conv<T>(x, w, bias, taps, y, d, layout, 0, st);
     if (tiled != -100) return tiled;
     const int nhwc = try_nhwc_conv<T, NHWC_FPROP>(x, w, bias, taps, y, d, layout, st);
     if (nhwc != -100) return nhwc;
@@ -231,6 +234,8 @@ int dgrad_t(const void *dy, const float *w, const void *taps, void *dx, const Co
     if (fast != -100) return fast;
     const int sliced = try_nhwc_plane_conv<T>(OP_DGRAD, dy, w, nullptr, taps, dx, d, layout, st);
     if (sliced != -100) return sliced;
+    const int tiled = try_tile_conv<T>(dy, w, nullptr, taps, dx, d, layout, 1, st);
+    if (tiled != -100) return tiled;
     const int nhwc = try_nhwc_conv<T, NHWC_DGRAD>(dy, w, nullptr, taps, dx, d, layout, st);
     if (nhwc != -100) return nhwc;
     const int total = d.N * d.C * d.H * d.W;

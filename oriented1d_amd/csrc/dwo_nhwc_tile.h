@@ -1,6 +1,8 @@
-// NHWC fprop for any plane extent and stride (channel count a multiple of 4): the stem
-// convolutions of the ConvNeXt-1D networks (224 -> 112 -> 56, stride 2) and every other NHWC
-// shape without compile-time planes.
+// fprop (and, with reversed weights, stride-1 dgrad) for any plane extent, stride and kernel
+// size: the stem convolutions of the ConvNeXt-1D networks (NHWC, 224 -> 112 -> 56, stride 2),
+// the stages of inputs other than 224 x 224 (NCHW), and every other shape without compile-time
+// planes.  NHWC needs a channel count that is a multiple of 4.  Described for NHWC; NCHW differs
+// only in how the window is loaded and the results are stored (PlaneSource).
 //
 // A workgroup owns four consecutive channels of a band of output rows of one image and walks
 // the band in sub-tiles.  Per sub-tile it loads the pixel slices of the input window (8 or 16
@@ -51,6 +53,7 @@ __device__ __forceinline__ void slice_load(Vec4<f16_t> &v, __amdgpu_buffer_rsrc_
 // output would be.
 template <typename T>
 struct SliceSource {
+    static constexpr bool kNchw = false;
     typedef Vec4<T> Payload;
     struct Params {
         const T *x;
@@ -71,6 +74,42 @@ struct SliceSource {
     __device__ __forceinline__ T elem(const Payload &v, int ch, bool) const { return v.elem(ch); }
 };
 
+__device__ __forceinline__ float buffer_value(__amdgpu_buffer_rsrc_t r, unsigned off, float);
+__device__ __forceinline__ float buffer_value(__amdgpu_buffer_rsrc_t r, unsigned off, bf16_t);
+__device__ __forceinline__ float buffer_value(__amdgpu_buffer_rsrc_t r, unsigned off, f16_t);
+
+// PlaneSource: an NCHW tensor; a pixel's payload is one element from each of the workgroup's
+// four channel planes (consecutive lanes read consecutive pixels of a row, so every plane's
+// loads are contiguous).  Channels beyond C (a last, partial group of four) read as zeros.
+template <typename T>
+struct PlaneSource {
+    static constexpr bool kNchw = true;
+    struct Payload {
+        float v[kSliceCh];
+    };
+    struct Params {
+        const T *x;
+    };
+    __amdgpu_buffer_rsrc_t img;
+    unsigned plane_bytes, c0_bytes;
+    __device__ __forceinline__ void init(const Params &p, int n, int c0, const ConvDims &d) {
+        const T *xn = p.x + (size_t)n * d.C * d.H * d.W;
+        img = __builtin_amdgcn_make_buffer_rsrc(
+            const_cast<T *>(xn), 0, (unsigned)((size_t)d.C * d.H * d.W * sizeof(T)), 0x00020000);
+        plane_bytes = (unsigned)(d.H * d.W) * (unsigned)sizeof(T);
+        c0_bytes = (unsigned)c0 * plane_bytes;
+    }
+    __device__ __forceinline__ void load(Payload &v, bool inside, unsigned pixel) const {
+#pragma unroll
+        for (int ch = 0; ch < kSliceCh; ch++)
+            v.v[ch] = buffer_value(
+                img, inside ? c0_bytes + ch * plane_bytes + pixel * (unsigned)sizeof(T) : 0xffffffffu, T{});
+    }
+    __device__ __forceinline__ T elem(const Payload &v, int ch, bool) const {
+        return from_float<T>(v.v[ch]);  // exact: the value came from a T
+    }
+};
+
 __device__ __forceinline__ float buffer_value(__amdgpu_buffer_rsrc_t r, unsigned off, float) {
     return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, off, 0, 0));
 }
@@ -83,6 +122,7 @@ __device__ __forceinline__ float buffer_value(__amdgpu_buffer_rsrc_t r, unsigned
 
 template <typename T, int CIN>
 struct PointwiseSource {
+    static constexpr bool kNchw = false;
     struct Payload {
         float v[CIN];
     };
@@ -126,7 +166,8 @@ __device__ __forceinline__ unsigned div_magic(unsigned d) {
 template <typename T, class Src>
 __global__ __launch_bounds__(kTileThreads) __attribute__((amdgpu_waves_per_eu(4, 4))) void nhwc_tile_fprop_kernel(
     typename Src::Params sp, const float *__restrict__ wt, const float *__restrict__ bias,
-    const int8_t *__restrict__ dhdw, T *__restrict__ y, ConvDims d, int nbands, int tasks_per_image) {
+    const int8_t *__restrict__ dhdw, T *__restrict__ y, ConvDims d, int nbands, int tasks_per_image,
+    int flip) {
     extern __shared__ float lds_f[];
     T *planes = reinterpret_cast<T *>(lds_f);
     float *lout = reinterpret_cast<float *>(planes + kSliceCh * kTilePlaneElems);
@@ -139,12 +180,12 @@ __global__ __launch_bounds__(kTileThreads) __attribute__((amdgpu_waves_per_eu(4,
     const int n = xcd + 8 * (local / tasks_per_image);
     if (n >= d.N) return;
     const int task = local % tasks_per_image;
-    const int nslices = d.C / kSliceCh;
+    const int nslices = (d.C + kSliceCh - 1) / kSliceCh;
     const int slice = task % nslices, band = task / nslices;
     const int c0 = slice * kSliceCh;
     const int sub = __builtin_amdgcn_readfirstlane(threadIdx.x / kTileSub);
     const unsigned stid = threadIdx.x % kTileSub;
-    const int c = c0 + sub;
+    const int c = min(c0 + sub, d.C - 1);  // (a partial last group repeats its last channel)
     const int s_ = d.stride, K = d.K;
 
     // tap extents of this sub-group's channel (uniform), then of the four channels together
@@ -196,9 +237,9 @@ __global__ __launch_bounds__(kTileThreads) __attribute__((amdgpu_waves_per_eu(4,
     int2 *mytab = tapt + sub * DWO_MAX_K;
     if ((int)stid < K)
         mytab[stid] = make_int2(((int)mytaps[2 * stid] / rstep) * iwp + (int)mytaps[2 * stid + 1] / cstep,
-                                __float_as_int(wt[(size_t)c * K + stid]));
+                                __float_as_int(wt[(size_t)c * K + (flip ? K - 1 - (int)stid : (int)stid)]));
 
-    T *yn = y + (size_t)n * d.P * d.Q * d.C + c0;
+    T *yn = Src::kNchw ? y + ((size_t)n * d.C + c0) * d.P * d.Q : y + (size_t)n * d.P * d.Q * d.C + c0;
     const T *plane = planes + sub * kTilePlaneElems;
     const unsigned nwin = ih * iw, nout = th * tw;
 
@@ -274,14 +315,26 @@ __global__ __launch_bounds__(kTileThreads) __attribute__((amdgpu_waves_per_eu(4,
                     if (o0 + k * kTileSub < nout) lout[sub * kTileOutputs + o0 + k * kTileSub] = acc[k];
             }
             __syncthreads();
-            for (unsigned o = threadIdx.x; o < nout; o += kTileThreads) {
-                const unsigned pl = fast_div(o, m_tw), ql = o - pl * tw;
-                const int p = pt + (int)pl, q = qt + (int)ql;
-                if (p < p_hi && q < d.Q) {
-                    Vec4<T> out;
-                    out.set(lout[o], lout[kTileOutputs + o], lout[2 * kTileOutputs + o],
-                            lout[3 * kTileOutputs + o]);
-                    out.store_cached(yn + ((size_t)p * d.Q + q) * d.C);
+            if constexpr (Src::kNchw) {
+                // rows of each channel plane: consecutive lanes, consecutive columns
+                const int nch = min(kSliceCh, d.C - c0);
+                for (unsigned i = threadIdx.x; i < nout * nch; i += kTileThreads) {
+                    const unsigned ch = i / nout, o = i - ch * nout;
+                    const unsigned pl = fast_div(o, m_tw), ql = o - pl * tw;
+                    const int p = pt + (int)pl, q = qt + (int)ql;
+                    if (p < p_hi && q < d.Q)
+                        yn[((size_t)ch * d.P + p) * d.Q + q] = from_float<T>(lout[ch * kTileOutputs + o]);
+                }
+            } else {
+                for (unsigned o = threadIdx.x; o < nout; o += kTileThreads) {
+                    const unsigned pl = fast_div(o, m_tw), ql = o - pl * tw;
+                    const int p = pt + (int)pl, q = qt + (int)ql;
+                    if (p < p_hi && q < d.Q) {
+                        Vec4<T> out;
+                        out.set(lout[o], lout[kTileOutputs + o], lout[2 * kTileOutputs + o],
+                                lout[3 * kTileOutputs + o]);
+                        out.store_cached(yn + ((size_t)p * d.Q + q) * d.C);
+                    }
                 }
             }
         }
@@ -291,7 +344,7 @@ __global__ __launch_bounds__(kTileThreads) __attribute__((amdgpu_waves_per_eu(4,
 // grid: 8 * ceil(N / 8) * bands * slices workgroups
 template <typename T, class Src>
 int launch_nhwc_tile(const typename Src::Params &sp, const float *w, const float *bias,
-                     const void *taps, void *y, const ConvDims &d, hipStream_t st) {
+                     const void *taps, void *y, const ConvDims &d, int flip, hipStream_t st) {
     const size_t lds = nhwc_tile_lds_bytes<T>();
     static const bool once = [&] {
         allow_large_lds(nhwc_tile_fprop_kernel<T, Src>, lds);
@@ -299,19 +352,25 @@ int launch_nhwc_tile(const typename Src::Params &sp, const float *w, const float
     }();
     (void)once;
     const int nbands = (d.P + kTileBandRows - 1) / kTileBandRows;
-    const int tpi = nbands * (d.C / kSliceCh);
+    const int tpi = nbands * ((d.C + kSliceCh - 1) / kSliceCh);
     const long grid = 8L * ((d.N + 7) / 8) * tpi;
     if (grid > 0x7fffffffL) return DWO_ERR_BAD_SHAPE;
     nhwc_tile_fprop_kernel<T, Src><<<dim3((unsigned)grid), dim3(kTileThreads), lds, st>>>(
-        sp, w, bias, taps_dhdw(taps), (T *)y, d, nbands, tpi);
+        sp, w, bias, taps_dhdw(taps), (T *)y, d, nbands, tpi, flip);
     const hipError_t e = hipGetLastError();
     return e == hipSuccess ? 0 : (int)e;
 }
 
+// flip = 1 reverses the weights: with stride 1 that is dgrad (the offsets are odd-symmetric)
 template <typename T>
 int launch_nhwc_tile_fprop(const void *x, const float *w, const float *bias, const void *taps,
-                           void *y, const ConvDims &d, hipStream_t st) {
-    return launch_nhwc_tile<T, SliceSource<T>>({(const T *)x}, w, bias, taps, y, d, st);
+                           void *y, const ConvDims &d, int flip, hipStream_t st) {
+    return launch_nhwc_tile<T, SliceSource<T>>({(const T *)x}, w, bias, taps, y, d, flip, st);
+}
+template <typename T>
+int launch_nchw_tile_fprop(const void *x, const float *w, const float *bias, const void *taps,
+                           void *y, const ConvDims &d, int flip, hipStream_t st) {
+    return launch_nhwc_tile<T, PlaneSource<T>>({(const T *)x}, w, bias, taps, y, d, flip, st);
 }
 
 // fprop of the C-channel tensor pw(x): x [N,H,W,CIN], pw_w [C,CIN], pw_b [C] or null
@@ -320,7 +379,7 @@ int launch_nhwc_tile_pointwise_fprop(const void *x, const float *pw_w, const flo
                                      const float *w, const float *bias, const void *taps, void *y,
                                      const ConvDims &d, hipStream_t st) {
     return launch_nhwc_tile<T, PointwiseSource<T, CIN>>({(const T *)x, pw_w, pw_b}, w, bias, taps, y,
-                                                         d, st);
+                                                         d, 0, st);
 }
 
 }  // namespace dwo
