@@ -157,15 +157,16 @@ int wgrad_max_partials(const ConvDims &d, int layout) {
     return nbatch < kMaxPlaneGroups ? nbatch : kMaxPlaneGroups;
 }
 
-// fprop (flip = 0) or stride-1 dgrad (flip = 1) at any extent by the tile kernel: NCHW always,
-// NHWC with the channel count a multiple of 4; images up to 4 GB (32-bit offsets inside one)
+// fprop (flip = 0) or dgrad (flip = 1) at any extent by the tile kernels: NCHW always, NHWC with
+// the channel count a multiple of 4; images below 2 GB (32-bit offsets inside one)
 template <typename T>
 int try_tile_conv(const void *x, const float *w, const float *bias, const void *taps, void *y,
                   const ConvDims &d, int layout, int flip, hipStream_t st) {
-    if (flip && d.stride != 1) return -100;
-    if ((size_t)d.H * d.W * d.C * sizeof(T) >= 0xffffffffull) return -100;
+    if ((size_t)d.H * d.W * d.C * sizeof(T) >= 0x80000000ull) return -100;
+    if (layout != DWO_NCHW && d.C % kSliceCh != 0) return -100;
+    if (flip && d.stride != 1)
+        return launch_tile_dgrad_strided<T>(x, w, taps, y, d, layout == DWO_NCHW, st);
     if (layout == DWO_NCHW) return launch_nchw_tile_fprop<T>(x, w, bias, taps, y, d, flip, st);
-    if (d.C % kSliceCh != 0) return -100;
     return launch_nhwc_tile_fprop<T>(x, w, bias, taps, y, d, flip, st);
 }
 

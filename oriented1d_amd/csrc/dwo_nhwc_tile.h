@@ -15,6 +15,8 @@
 // K / 2 in each direction, whatever the angles.
 #pragma once
 
+#include <type_traits>
+
 #include "dwo_static.h"
 
 namespace dwo {
@@ -24,7 +26,7 @@ constexpr int kTileSub = kTileThreads / kSliceCh;          // threads per channe
 constexpr int kTilePlaneElems = 7680;                      // LDS elements per channel plane (two
                                                            // workgroups of 16-bit planes per CU)
 constexpr int kTileOutputs = 1024;                         // most outputs per sub-tile
-constexpr int kTileBandRows = 32;                          // output rows per workgroup
+constexpr int kTileBandRows = 32;                          // most output rows per workgroup
 
 // planes, fp32 results, per-channel tap table (offset, weight) and tap extents
 template <typename T>
@@ -74,40 +76,61 @@ struct SliceSource {
     __device__ __forceinline__ T elem(const Payload &v, int ch, bool) const { return v.elem(ch); }
 };
 
-__device__ __forceinline__ float buffer_value(__amdgpu_buffer_rsrc_t r, unsigned off, float);
-__device__ __forceinline__ float buffer_value(__amdgpu_buffer_rsrc_t r, unsigned off, bf16_t);
-__device__ __forceinline__ float buffer_value(__amdgpu_buffer_rsrc_t r, unsigned off, f16_t);
-
 // PlaneSource: an NCHW tensor; a pixel's payload is one element from each of the workgroup's
 // four channel planes (consecutive lanes read consecutive pixels of a row, so every plane's
 // loads are contiguous).  Channels beyond C (a last, partial group of four) read as zeros.
+// one element from each of four planes: fp32 as they are, 16-bit types packed in pairs
+template <typename T>
+struct PlanePixels {
+    unsigned v[kSliceCh / 2];
+    __device__ __forceinline__ void load(__amdgpu_buffer_rsrc_t r, unsigned off, unsigned plane_bytes) {
+#pragma unroll
+        for (int k = 0; k < kSliceCh / 2; k++) {
+            const unsigned lo = (uint16_t)__builtin_amdgcn_raw_buffer_load_b16(r, off, 0, 0);
+            const unsigned hi = (uint16_t)__builtin_amdgcn_raw_buffer_load_b16(r, off + plane_bytes, 0, 0);
+            v[k] = lo | hi << 16;
+            off += 2 * plane_bytes;
+        }
+    }
+    __device__ __forceinline__ T elem(int ch) const {
+        return __builtin_bit_cast(T, (uint16_t)(v[ch / 2] >> (16 * (ch % 2))));
+    }
+};
+template <>
+struct PlanePixels<float> {
+    float v[kSliceCh];
+    __device__ __forceinline__ void load(__amdgpu_buffer_rsrc_t r, unsigned off, unsigned plane_bytes) {
+#pragma unroll
+        for (int k = 0; k < kSliceCh; k++)
+            v[k] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, off + k * plane_bytes, 0, 0));
+    }
+    __device__ __forceinline__ float elem(int ch) const { return v[ch]; }
+};
+
+// PlaneSource: an NCHW tensor; a pixel's payload is one element from each of the workgroup's
+// four channel planes (consecutive lanes read consecutive pixels of a row, so every plane's
+// loads are contiguous).  Channels beyond C (a last, partial group of four) read as zeros: the
+// descriptor ends with the image.
 template <typename T>
 struct PlaneSource {
     static constexpr bool kNchw = true;
-    struct Payload {
-        float v[kSliceCh];
-    };
+    typedef PlanePixels<T> Payload;
     struct Params {
         const T *x;
     };
     __amdgpu_buffer_rsrc_t img;
-    unsigned plane_bytes, c0_bytes;
+    unsigned plane_bytes;
     __device__ __forceinline__ void init(const Params &p, int n, int c0, const ConvDims &d) {
-        const T *xn = p.x + (size_t)n * d.C * d.H * d.W;
+        const T *xn = p.x + ((size_t)n * d.C + c0) * d.H * d.W;
         img = __builtin_amdgcn_make_buffer_rsrc(
-            const_cast<T *>(xn), 0, (unsigned)((size_t)d.C * d.H * d.W * sizeof(T)), 0x00020000);
+            const_cast<T *>(xn), 0, (unsigned)((size_t)(d.C - c0) * d.H * d.W * sizeof(T)), 0x00020000);
         plane_bytes = (unsigned)(d.H * d.W) * (unsigned)sizeof(T);
-        c0_bytes = (unsigned)c0 * plane_bytes;
     }
     __device__ __forceinline__ void load(Payload &v, bool inside, unsigned pixel) const {
-#pragma unroll
-        for (int ch = 0; ch < kSliceCh; ch++)
-            v.v[ch] = buffer_value(
-                img, inside ? c0_bytes + ch * plane_bytes + pixel * (unsigned)sizeof(T) : 0xffffffffu, T{});
+        // (an offset that stays beyond the descriptor after the three plane steps)
+        v.load(img, inside ? pixel * (unsigned)sizeof(T) : 0x80000000u, plane_bytes);
     }
-    __device__ __forceinline__ T elem(const Payload &v, int ch, bool) const {
-        return from_float<T>(v.v[ch]);  // exact: the value came from a T
-    }
+    __device__ __forceinline__ T elem(const Payload &v, int ch, bool) const { return v.elem(ch); }
 };
 
 __device__ __forceinline__ float buffer_value(__amdgpu_buffer_rsrc_t r, unsigned off, float) {
@@ -163,10 +186,46 @@ __device__ __forceinline__ unsigned div_magic(unsigned d) {
     return (unsigned)((0x100000000ull + d - 1) / d);
 }
 
+// Results of a th x tw sub-tile at (pt, qt), one fp32 plane of `stride` floats per channel in
+// `lout`, to the image at `yn` (rows below p_hi, columns below Q): NCHW as rows of each channel
+// plane (consecutive lanes, consecutive columns), NHWC as four-channel pixel slices.
+template <typename T, bool NCHW>
+__device__ __forceinline__ void tile_flush(const float *lout, int stride, T *yn, unsigned nout,
+                                           unsigned tw, unsigned m_tw, int pt, int qt, int p_hi, int P,
+                                           int Q, int C, int c0) {
+    if constexpr (NCHW) {
+        const int nch = min(kSliceCh, C - c0);
+        for (int ch = 0; ch < nch; ch++)
+            for (unsigned o = threadIdx.x; o < nout; o += kTileThreads) {
+                const unsigned pl = fast_div(o, m_tw), ql = o - pl * tw;
+                const int p = pt + (int)pl, q = qt + (int)ql;
+                if (p < p_hi && q < Q)
+                    yn[((size_t)ch * P + p) * Q + q] = from_float<T>(lout[ch * stride + o]);
+            }
+    } else {
+        for (unsigned o = threadIdx.x; o < nout; o += kTileThreads) {
+            const unsigned pl = fast_div(o, m_tw), ql = o - pl * tw;
+            const int p = pt + (int)pl, q = qt + (int)ql;
+            if (p < p_hi && q < Q) {
+                Vec4<T> out;
+                out.set(lout[o], lout[stride + o], lout[2 * stride + o], lout[3 * stride + o]);
+                out.store_cached(yn + ((size_t)p * Q + q) * C);
+            }
+        }
+    }
+}
+
+// Rows per band: 32, fewer while the grid would not fill the chip's workgroup slots twice.
+inline int tile_band_rows(int N, int rows, int nslices) {
+    int band = kTileBandRows;
+    while (band > 8 && (long)N * ((rows + band - 1) / band) * nslices < 1024) band /= 2;
+    return band;
+}
+
 template <typename T, class Src>
 __global__ __launch_bounds__(kTileThreads) __attribute__((amdgpu_waves_per_eu(4, 4))) void nhwc_tile_fprop_kernel(
     typename Src::Params sp, const float *__restrict__ wt, const float *__restrict__ bias,
-    const int8_t *__restrict__ dhdw, T *__restrict__ y, ConvDims d, int nbands, int tasks_per_image,
+    const int8_t *__restrict__ dhdw, T *__restrict__ y, ConvDims d, int nbands, int band_rows,
     int flip) {
     extern __shared__ float lds_f[];
     T *planes = reinterpret_cast<T *>(lds_f);
@@ -174,14 +233,14 @@ __global__ __launch_bounds__(kTileThreads) __attribute__((amdgpu_waves_per_eu(4,
     int2 *tapt = reinterpret_cast<int2 *>(lout + kSliceCh * kTileOutputs);  // [ch][K] (offset, weight)
     int *halo = reinterpret_cast<int *>(tapt + kSliceCh * DWO_MAX_K);       // [ch][2]
 
-    // image n of XCD n % 8: hardware deals consecutive workgroup ids to the XCDs in turn, so the
-    // slices and bands of one image share one L2
-    const int xcd = blockIdx.x % 8, local = blockIdx.x / 8;
-    const int n = xcd + 8 * (local / tasks_per_image);
-    if (n >= d.N) return;
-    const int task = local % tasks_per_image;
+    // Unit (image, band) u runs on XCD u % 8: hardware deals consecutive workgroup ids to the
+    // XCDs in turn, so the slices of one band (which share every cache line they touch, NHWC)
+    // meet in one L2.
     const int nslices = (d.C + kSliceCh - 1) / kSliceCh;
-    const int slice = task % nslices, band = task / nslices;
+    const int unit = blockIdx.x % 8 + 8 * (blockIdx.x / 8 / nslices);
+    if (unit >= d.N * nbands) return;
+    const int slice = blockIdx.x / 8 % nslices;
+    const int n = unit / nbands, band = unit - n * nbands;
     const int c0 = slice * kSliceCh;
     const int sub = __builtin_amdgcn_readfirstlane(threadIdx.x / kTileSub);
     const unsigned stid = threadIdx.x % kTileSub;
@@ -211,7 +270,7 @@ __global__ __launch_bounds__(kTileThreads) __attribute__((amdgpu_waves_per_eu(4,
     // sub-tile shape: th rows x tw columns of outputs; window ih x iw of inputs.  Cost per
     // output = window positions plus a fixed per-sub-tile charge (barriers, pipeline fill).
     // (widths of at least 2, also for a one-column plane: the index arithmetic divides by them)
-    const int p_lo = band * kTileBandRows, p_hi = min(d.P, p_lo + kTileBandRows);
+    const int p_lo = band * band_rows, p_hi = min(d.P, p_lo + band_rows);
     const int RH = p_hi - p_lo;
     const int Qe = max(d.Q, 2);
     int th = 1, tw = 2;
@@ -315,33 +374,13 @@ __global__ __launch_bounds__(kTileThreads) __attribute__((amdgpu_waves_per_eu(4,
                     if (o0 + k * kTileSub < nout) lout[sub * kTileOutputs + o0 + k * kTileSub] = acc[k];
             }
             __syncthreads();
-            if constexpr (Src::kNchw) {
-                // rows of each channel plane: consecutive lanes, consecutive columns
-                const int nch = min(kSliceCh, d.C - c0);
-                for (unsigned i = threadIdx.x; i < nout * nch; i += kTileThreads) {
-                    const unsigned ch = i / nout, o = i - ch * nout;
-                    const unsigned pl = fast_div(o, m_tw), ql = o - pl * tw;
-                    const int p = pt + (int)pl, q = qt + (int)ql;
-                    if (p < p_hi && q < d.Q)
-                        yn[((size_t)ch * d.P + p) * d.Q + q] = from_float<T>(lout[ch * kTileOutputs + o]);
-                }
-            } else {
-                for (unsigned o = threadIdx.x; o < nout; o += kTileThreads) {
-                    const unsigned pl = fast_div(o, m_tw), ql = o - pl * tw;
-                    const int p = pt + (int)pl, q = qt + (int)ql;
-                    if (p < p_hi && q < d.Q) {
-                        Vec4<T> out;
-                        out.set(lout[o], lout[kTileOutputs + o], lout[2 * kTileOutputs + o],
-                                lout[3 * kTileOutputs + o]);
-                        out.store_cached(yn + ((size_t)p * d.Q + q) * d.C);
-                    }
-                }
-            }
+            tile_flush<T, Src::kNchw>(lout, kTileOutputs, yn, nout, tw, m_tw, pt, qt, p_hi, d.P, d.Q, d.C,
+                                      c0);
         }
     }
 }
 
-// grid: 8 * ceil(N / 8) * bands * slices workgroups
+// grid: 8 * ceil(N * bands / 8) * slices workgroups
 template <typename T, class Src>
 int launch_nhwc_tile(const typename Src::Params &sp, const float *w, const float *bias,
                      const void *taps, void *y, const ConvDims &d, int flip, hipStream_t st) {
@@ -351,12 +390,13 @@ int launch_nhwc_tile(const typename Src::Params &sp, const float *w, const float
         return true;
     }();
     (void)once;
-    const int nbands = (d.P + kTileBandRows - 1) / kTileBandRows;
-    const int tpi = nbands * ((d.C + kSliceCh - 1) / kSliceCh);
-    const long grid = 8L * ((d.N + 7) / 8) * tpi;
+    const int nslices = (d.C + kSliceCh - 1) / kSliceCh;
+    const int band_rows = tile_band_rows(d.N, d.P, nslices);
+    const int nbands = (d.P + band_rows - 1) / band_rows;
+    const long grid = 8L * (((long)d.N * nbands + 7) / 8) * nslices;
     if (grid > 0x7fffffffL) return DWO_ERR_BAD_SHAPE;
     nhwc_tile_fprop_kernel<T, Src><<<dim3((unsigned)grid), dim3(kTileThreads), lds, st>>>(
-        sp, w, bias, taps_dhdw(taps), (T *)y, d, nbands, tpi, flip);
+        sp, w, bias, taps_dhdw(taps), (T *)y, d, nbands, band_rows, flip);
     const hipError_t e = hipGetLastError();
     return e == hipSuccess ? 0 : (int)e;
 }
@@ -380,6 +420,237 @@ int launch_nhwc_tile_pointwise_fprop(const void *x, const float *pw_w, const flo
                                      const ConvDims &d, hipStream_t st) {
     return launch_nhwc_tile<T, PointwiseSource<T, CIN>>({(const T *)x, pw_w, pw_b}, w, bias, taps, y,
                                                          d, 0, st);
+}
+
+// ---------------------------------------------------------------------------------------------
+// dgrad with stride 2 or 4 (ops.py:64-88 with the strides of models/convnext.py:141-150).
+// dx(h, w) sums w_t * dy((h - dh_t) / s, (w - dw_t) / s) over the taps t whose offsets have h's
+// and w's residues modulo s.  The dx pixels of one residue class (a, b) therefore are a
+// stride-1 gather over dy with that class's taps at offsets (-floor(dh_t / s), -floor(dw_t / s)),
+// and every tap belongs to exactly one class: 1 / s^2 of the multiply-adds of a gather that
+// tests all taps at every pixel.  A workgroup owns four channels of a band of dx rows; per
+// sub-tile it stages the dy window as one plane per channel in LDS, lets sub-group k evaluate
+// channel k class after class (its tap table is sorted by class), places the sums at their dx
+// positions in LDS and writes the sub-tile out in raster order.
+constexpr int kDgradPlaneElems = 4096;  // LDS elements per channel plane (dy window)
+constexpr int kDgradOutputs = 2048;     // most dx pixels per sub-tile
+constexpr int kDgradClasses = 16;       // residue classes at stride 4
+
+template <typename T>
+constexpr size_t tile_dgrad_lds_bytes() {
+    return (size_t)kSliceCh * kDgradPlaneElems * sizeof(T) + (size_t)kSliceCh * kDgradOutputs * 4 +
+           (size_t)kSliceCh * DWO_MAX_K * 8 + (size_t)kSliceCh * (kDgradClasses + 1) * 4 + 64;
+}
+
+template <typename T, class Src>
+__global__ __launch_bounds__(kTileThreads) __attribute__((amdgpu_waves_per_eu(4, 4))) void tile_dgrad_strided_kernel(
+    typename Src::Params sp, const float *__restrict__ wt, const int8_t *__restrict__ dhdw,
+    T *__restrict__ dx, ConvDims d, int nbands, int band_rows) {
+    extern __shared__ float lds_f[];
+    T *planes = reinterpret_cast<T *>(lds_f);
+    float *lout = reinterpret_cast<float *>(planes + kSliceCh * kDgradPlaneElems);
+    int2 *tapt = reinterpret_cast<int2 *>(lout + kSliceCh * kDgradOutputs);  // [ch][K], by class
+    int *cstart = reinterpret_cast<int *>(tapt + kSliceCh * DWO_MAX_K);     // [ch][classes + 1]
+    int *halo = cstart + kSliceCh * (kDgradClasses + 1);                    // [ch][2]
+
+    const int nslices = (d.C + kSliceCh - 1) / kSliceCh;
+    const int unit = blockIdx.x % 8 + 8 * (blockIdx.x / 8 / nslices);
+    if (unit >= d.N * nbands) return;
+    const int slice = blockIdx.x / 8 % nslices;
+    const int n = unit / nbands, band = unit - n * nbands;
+    const int c0 = slice * kSliceCh;
+    const int sub = __builtin_amdgcn_readfirstlane(threadIdx.x / kTileSub);
+    const unsigned stid = threadIdx.x % kTileSub;
+    const int c = min(c0 + sub, d.C - 1);
+    const int s_ = d.stride, sh = d.shift, K = d.K, ncls = s_ * s_;
+
+    // tap t: residue class and offset in dy
+    const int8_t *mytaps = dhdw + (size_t)c * K * 2;
+    auto tap_class = [&](int t, int &eh, int &ew) {
+        const int dh = mytaps[2 * t], dw = mytaps[2 * t + 1];
+        eh = -(dh >> sh), ew = -(dw >> sh);  // (arithmetic shifts: floor)
+        return (dh & (s_ - 1)) * s_ + (dw & (s_ - 1));
+    };
+    int hh = 0, hw = 0;
+    for (int t = 0; t < K; t++) {
+        int eh, ew;
+        tap_class(t, eh, ew);
+        hh = max(hh, abs(eh));
+        hw = max(hw, abs(ew));
+    }
+    if (stid == 0) halo[sub * 2] = hh, halo[sub * 2 + 1] = hw;
+    __syncthreads();
+    hh = max(max(halo[0], halo[2]), max(halo[4], halo[6]));
+    hw = max(max(halo[1], halo[3]), max(halo[5], halo[7]));
+    hh = __builtin_amdgcn_readfirstlane(hh);
+    hw = __builtin_amdgcn_readfirstlane(hw);
+
+    // sub-tile: th x tw dx pixels (multiples of the stride), window ih x iw of dy
+    const int h_lo = band * band_rows, h_hi = min(d.H, h_lo + band_rows);
+    const int RH = (h_hi - h_lo + s_ - 1) & ~(s_ - 1);
+    const int We = max((d.W + s_ - 1) & ~(s_ - 1), 2 * s_);
+    int th = s_, tw = 8;
+    {
+        float best = 1e30f;
+        for (int a = RH;; a = (((a + 1) / 2) + s_ - 1) & ~(s_ - 1)) {
+            for (int k = -1; k < 6; k++) {
+                const int b = k < 0 ? We : (256 >> k);  // full width, 256, 128, 64, 32, 16, 8
+                if (b > We || a * b > kDgradOutputs) continue;
+                const int ih = (a >> sh) + 2 * hh, iw = ((b >> sh) + 2 * hw) | 1;
+                if (ih * iw > kDgradPlaneElems) continue;
+                const float cost = (float)(ih * iw + 1536) / (float)(a * b);
+                if (cost < best) best = cost, th = a, tw = b;
+            }
+            if (a <= s_) break;
+        }
+    }
+    const int csh = th >> sh, csw = tw >> sh;  // a class's pixels in the sub-tile
+    const int ih = csh + 2 * hh, iw = csw + 2 * hw, iwp = iw | 1;
+    const unsigned m_iw = div_magic(iw), m_tw = div_magic(tw), m_csw = div_magic(csw);
+    const unsigned nwin = ih * iw, nout = th * tw, csz = csh * csw;
+
+    // the channel's taps sorted by class as (LDS element offset, weight), and the class ranges
+    int2 *mytab = tapt + sub * DWO_MAX_K;
+    int *mystart = cstart + sub * (kDgradClasses + 1);
+    if ((int)stid < K) {
+        int eh, ew, fh, fw;
+        const int cls = tap_class(stid, eh, ew);
+        int rank = 0;
+        for (int t = 0; t < K; t++) {
+            const int other = tap_class(t, fh, fw);
+            rank += (other < cls || (other == cls && t < (int)stid)) ? 1 : 0;
+        }
+        mytab[rank] = make_int2(eh * iwp + ew, __float_as_int(wt[(size_t)c * K + stid]));
+    }
+    if ((int)stid <= ncls) {
+        int below = 0, fh, fw;
+        for (int t = 0; t < K; t++) below += tap_class(t, fh, fw) < (int)stid ? 1 : 0;
+        mystart[stid] = below;
+    }
+
+    T *dxn = Src::kNchw ? dx + ((size_t)n * d.C + c0) * d.H * d.W : dx + (size_t)n * d.H * d.W * d.C + c0;
+    const T *plane = planes + sub * kDgradPlaneElems;
+    float *myout = lout + sub * kDgradOutputs;
+
+    constexpr int PRE = kDgradPlaneElems / kTileThreads;
+    typename Src::Payload pre[PRE];
+    Src source;
+    ConvDims ds = d;  // the source tensor is dy: P x Q
+    ds.H = d.P, ds.W = d.Q;
+    source.init(sp, n, c0, ds);
+    auto window_pixel = [&](int ht, int wt_, unsigned v, unsigned &pixel) {
+        const unsigned i = fast_div(v, m_iw), j = v - i * iw;
+        const unsigned r = (unsigned)((ht >> sh) - hh + (int)i);
+        const unsigned q = (unsigned)((wt_ >> sh) - hw + (int)j);
+        pixel = r * d.Q + q;
+        return v < nwin && r < (unsigned)d.P && q < (unsigned)d.Q;
+    };
+    auto load_window = [&](int ht, int wt_) {
+#pragma unroll
+        for (int u = 0; u < PRE; u++) {
+            if (u * kTileThreads >= (int)nwin) break;
+            unsigned v = u * kTileThreads + threadIdx.x;
+            asm volatile("" : "+v"(v));
+            unsigned pixel;
+            const bool inside = window_pixel(ht, wt_, v, pixel);
+            source.load(pre[u], inside, pixel);
+        }
+    };
+    // R pixels of class (a, b) per thread, 128 apart in the class's raster order
+    auto eval = [&](auto rc, unsigned e0, int a, int b, int t0, int t1) {
+        constexpr int R = decltype(rc)::value;
+        const T *base[R];
+        float acc[R];
+        unsigned at[R];
+#pragma unroll
+        for (int k = 0; k < R; k++) {
+            const unsigned e = min(e0 + k * kTileSub, csz - 1);
+            const unsigned i = fast_div(e, m_csw), j = e - i * csw;
+            base[k] = plane + ((i + hh) * iwp + j + hw);
+            at[k] = ((i << sh) + a) * tw + (j << sh) + b;
+            acc[k] = 0.f;
+        }
+#pragma unroll 4
+        for (int t = t0; t < t1; t++) {
+            const int2 tp = mytab[t];
+            const float w = __int_as_float(tp.y);
+#pragma unroll
+            for (int k = 0; k < R; k++) acc[k] = __builtin_fmaf(to_float(base[k][tp.x]), w, acc[k]);
+        }
+#pragma unroll
+        for (int k = 0; k < R; k++)
+            if (e0 + k * kTileSub < csz) myout[at[k]] = acc[k];
+    };
+
+    load_window(h_lo, 0);
+    for (int ht = h_lo; ht < h_hi; ht += th) {
+        for (int wt_ = 0; wt_ < d.W; wt_ += tw) {
+#pragma unroll
+            for (int u = 0; u < PRE; u++) {
+                if (u * kTileThreads >= (int)nwin) break;
+                unsigned v = u * kTileThreads + threadIdx.x;
+                asm volatile("" : "+v"(v));
+                if (v < nwin) {
+                    const unsigned i = fast_div(v, m_iw), j = v - i * iw;
+                    const unsigned at = i * iwp + j;
+                    unsigned pixel;
+                    const bool inside = window_pixel(ht, wt_, v, pixel);
+#pragma unroll
+                    for (int ch = 0; ch < kSliceCh; ch++)
+                        planes[ch * kDgradPlaneElems + at] = source.elem(pre[u], ch, inside);
+                }
+            }
+            __syncthreads();
+            if (wt_ + tw < d.W)
+                load_window(ht, wt_ + tw);
+            else if (ht + th < h_hi)
+                load_window(ht + th, 0);
+            for (int cls = 0; cls < ncls; cls++) {
+                const int t0 = __builtin_amdgcn_readfirstlane(mystart[cls]);
+                const int t1 = __builtin_amdgcn_readfirstlane(mystart[cls + 1]);
+                const int a = cls >> sh, b = cls & (s_ - 1);
+                if (csz > 2 * kTileSub)
+                    for (unsigned e0 = stid; e0 < csz; e0 += 4 * kTileSub)
+                        eval(std::integral_constant<int, 4>{}, e0, a, b, t0, t1);
+                else if (csz > kTileSub)
+                    for (unsigned e0 = stid; e0 < csz; e0 += 2 * kTileSub)
+                        eval(std::integral_constant<int, 2>{}, e0, a, b, t0, t1);
+                else if (stid < csz)
+                    eval(std::integral_constant<int, 1>{}, stid, a, b, t0, t1);
+            }
+            __syncthreads();
+            tile_flush<T, Src::kNchw>(lout, kDgradOutputs, dxn, nout, tw, m_tw, ht, wt_, h_hi, d.H, d.W,
+                                      d.C, c0);
+        }
+    }
+}
+
+template <typename T, class Src>
+int launch_tile_dgrad_strided_src(const void *dy, const float *w, const void *taps, void *dx,
+                                  const ConvDims &d, hipStream_t st) {
+    const size_t lds = tile_dgrad_lds_bytes<T>();
+    static const bool once = [&] {
+        allow_large_lds(tile_dgrad_strided_kernel<T, Src>, lds);
+        return true;
+    }();
+    (void)once;
+    const int nslices = (d.C + kSliceCh - 1) / kSliceCh;
+    const int band_rows = tile_band_rows(d.N, d.H, nslices);
+    const int nbands = (d.H + band_rows - 1) / band_rows;
+    const long grid = 8L * (((long)d.N * nbands + 7) / 8) * nslices;
+    if (grid > 0x7fffffffL) return DWO_ERR_BAD_SHAPE;
+    tile_dgrad_strided_kernel<T, Src><<<dim3((unsigned)grid), dim3(kTileThreads), lds, st>>>(
+        {(const T *)dy}, w, taps_dhdw(taps), (T *)dx, d, nbands, band_rows);
+    const hipError_t e = hipGetLastError();
+    return e == hipSuccess ? 0 : (int)e;
+}
+
+// dgrad at stride 2 or 4: dy [N,C,P,Q] or [N,P,Q,C] -> dx [N,C,H,W] or [N,H,W,C]
+template <typename T>
+int launch_tile_dgrad_strided(const void *dy, const float *w, const void *taps, void *dx,
+                              const ConvDims &d, bool nchw, hipStream_t st) {
+    return nchw ? launch_tile_dgrad_strided_src<T, PlaneSource<T>>(dy, w, taps, dx, d, st)
+                : launch_tile_dgrad_strided_src<T, SliceSource<T>>(dy, w, taps, dx, d, st);
 }
 
 }  // namespace dwo

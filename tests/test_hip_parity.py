@@ -136,6 +136,17 @@ def test_nhwc_large_planes_many_tiles(oracle, stride, H, W, K, dtype):
     _case(oracle, 2, 36, H, W, K, stride, dtype, True, theta, seed=H + W + K)
 
 
+@pytest.mark.parametrize("dtype", DTYPES, ids=["f32", "bf16", "f16"])
+@pytest.mark.parametrize("stride,H,W,K", [(2, 150, 138, 31), (1, 70, 200, 15), (4, 97, 64, 27),
+                                          (2, 61, 35, 31)])
+def test_nchw_large_planes_many_tiles(oracle, stride, H, W, K, dtype):
+    """NCHW planes without compile-time kernels, several bands and sub-tiles per workgroup, a
+    channel count that leaves a partial last group of four; strided dgrad by residue classes."""
+    theta = np.concatenate([np.repeat(canonical_theta(8), 4),
+                            np.array([0.3, 1.1, 2.0, 2.9, 4.4, -0.7], dtype=np.float32)]).astype(np.float32)
+    _case(oracle, 3, 38, H, W, K, stride, dtype, False, theta, seed=H + W + K + 1)
+
+
 @pytest.mark.parametrize("nhwc", [False, True], ids=["nchw", "nhwc"])
 def test_random_angles_ragged_shapes(oracle, nhwc):
     rng = np.random.default_rng(77)
