@@ -141,13 +141,24 @@ int try_nhwc_plane_wgrad(const void *x, const void *dy, const void *taps, float 
     return -100;
 }
 
-int wgrad_max_partials(const ConvDims &d, int layout) {
+// shapes the tile kernels take: NCHW always, NHWC with the channel count a multiple of 4; images
+// below 2 GB (32-bit offsets inside one)
+bool tile_covers(const ConvDims &d, int layout, size_t esize) {
+    if ((size_t)d.H * d.W * d.C * esize >= 0x80000000ull) return false;
+    return layout == DWO_NCHW || d.C % kSliceCh == 0;
+}
+
+int wgrad_max_partials(const ConvDims &d, int layout, size_t esize) {
     const int PBI = nhwc_plane_batch(d, layout);
     if (PBI != 0) {
         const int nbatch = (d.N + PBI - 1) / PBI;
         return nbatch < kMaxPlaneGroups ? nbatch : kMaxPlaneGroups;
     }
     const int PB = plane_batch(d, layout);
+    if (PB == 0 && tile_covers(d, layout, esize)) {
+        int band_rows, nbands;
+        return tile_wgrad_groups(d, &band_rows, &nbands);
+    }
     if (PB == 0 && layout == DWO_NHWC && nhwc_has_k(d.K)) {
         int ppw = 0;
         return nhwc_wgrad_groups((long)d.N * d.P * d.Q, (d.C + 63) / 64, &ppw);
@@ -162,8 +173,7 @@ int wgrad_max_partials(const ConvDims &d, int layout) {
 template <typename T>
 int try_tile_conv(const void *x, const float *w, const float *bias, const void *taps, void *y,
                   const ConvDims &d, int layout, int flip, hipStream_t st) {
-    if ((size_t)d.H * d.W * d.C * sizeof(T) >= 0x80000000ull) return -100;
-    if (layout != DWO_NCHW && d.C % kSliceCh != 0) return -100;
+    if (!tile_covers(d, layout, sizeof(T))) return -100;
     if (flip && d.stride != 1)
         return launch_tile_dgrad_strided<T>(x, w, taps, y, d, layout == DWO_NCHW, st);
     if (layout == DWO_NCHW) return launch_nchw_tile_fprop<T>(x, w, bias, taps, y, d, flip, st);
@@ -263,6 +273,8 @@ int wgrad_t(const void *dy, const void *x, const void *taps, float *dw, float *d
     } else if (nhwc_plane_batch(d, layout) != 0) {
         rc = try_nhwc_plane_wgrad<T>(x, dy, taps, part, dw, db, &NG, d, st);
         direct = NG == 1;
+    } else if (tile_covers(d, layout, sizeof(T))) {
+        rc = launch_tile_wgrad<T>(x, dy, taps, part, &NG, d, layout == DWO_NCHW, st);
     } else if (layout == DWO_NHWC && nhwc_has_k(d.K)) {
         rc = try_nhwc_wgrad<T>(dy, x, taps, part, &NG, d, st);
     } else {
@@ -417,7 +429,7 @@ size_t dwo_wgrad_scratch_bytes(int N, int C, int H, int W, int K, int stride, in
                                int layout) {
     if (check_common(N, C, H, W, K, stride, dtype, layout) != DWO_OK) return 0;
     const ConvDims d = make_dims(N, C, H, W, K, stride);
-    return (size_t)C * (K + 1) * wgrad_max_partials(d, layout) * sizeof(float);
+    return (size_t)C * (K + 1) * wgrad_max_partials(d, layout, dtype == DWO_F32 ? 4 : 2) * sizeof(float);
 }
 
 int dwo_wgrad(const void *dy, const void *x, const void *taps, float *dw, float *db,

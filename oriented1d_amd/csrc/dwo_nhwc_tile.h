@@ -215,6 +215,28 @@ __device__ __forceinline__ void tile_flush(const float *lout, int stride, T *yn,
     }
 }
 
+// Sub-tile shape for a band of RH output rows: th rows x tw columns of outputs with a window
+// of ((th-1)*srow + 1 + 2*hh) x ((tw-1)*scol + 1 + 2*hw) inputs.  Cost per output = window
+// positions plus a fixed per-sub-tile charge (barriers, pipeline fill), compared as integer
+// cross products.  Widths: the full width `wfull` or a power of two from 8 to 128; widths of at
+// least 2, also for a one-column plane: the index arithmetic divides by them.
+__device__ __forceinline__ void choose_tile(int RH, int wfull, int srow, int scol, int hh, int hw,
+                                            int &th, int &tw) {
+    th = 1, tw = min(wfull, 8);
+    int best_num = 0x7fffffff / kTileOutputs, best_den = 1;
+    for (int a = RH; a >= 1; a = (a + 1) / 2) {
+        for (int k = 0; k < 6; k++) {
+            const int b = k == 0 ? wfull : (256 >> k);
+            if (b > wfull || a * b > kTileOutputs) continue;
+            const int ih = (a - 1) * srow + 1 + 2 * hh, iw = ((b - 1) * scol + 1 + 2 * hw) | 1;
+            if (ih * iw > kTilePlaneElems) continue;
+            const int num = ih * iw + 1536, den = a * b;
+            if (num * best_den < best_num * den) best_num = num, best_den = den, th = a, tw = b;
+        }
+        if (a == 1) break;
+    }
+}
+
 // Rows per band: 32, fewer while the grid would not fill the chip's workgroup slots twice.
 inline int tile_band_rows(int N, int rows, int nslices) {
     int band = kTileBandRows;
@@ -273,21 +295,8 @@ __global__ __launch_bounds__(kTileThreads) __attribute__((amdgpu_waves_per_eu(4,
     const int p_lo = band * band_rows, p_hi = min(d.P, p_lo + band_rows);
     const int RH = p_hi - p_lo;
     const int Qe = max(d.Q, 2);
-    int th = 1, tw = 2;
-    {
-        float best = 1e30f;
-        for (int a = RH; a >= 1; a = (a + 1) / 2) {
-            for (int k = 0; k < 6; k++) {
-                const int b = k == 0 ? Qe : (256 >> k);  // full width, 128, 64, 32, 16, 8
-                if (b > Qe || a * b > kTileOutputs) continue;
-                const int ih = (a - 1) * srow + 1 + 2 * hh, iw = ((b - 1) * scol + 1 + 2 * hw) | 1;
-                if (ih * iw > kTilePlaneElems) continue;
-                const float cost = (float)(ih * iw + 1536) / (float)(a * b);
-                if (cost < best) best = cost, th = a, tw = b;
-            }
-            if (a == 1) break;
-        }
-    }
+    int th, tw;
+    choose_tile(RH, Qe, srow, scol, hh, hw, th, tw);
     const int ih = (th - 1) * srow + 1 + 2 * hh;
     const int iw = (tw - 1) * scol + 1 + 2 * hw;
     const int iwp = iw | 1;
@@ -651,6 +660,235 @@ int launch_tile_dgrad_strided(const void *dy, const float *w, const void *taps, 
                               const ConvDims &d, bool nchw, hipStream_t st) {
     return nchw ? launch_tile_dgrad_strided_src<T, PlaneSource<T>>(dy, w, taps, dx, d, st)
                 : launch_tile_dgrad_strided_src<T, SliceSource<T>>(dy, w, taps, dx, d, st);
+}
+
+// ---------------------------------------------------------------------------------------------
+// wgrad for any plane extent, stride and kernel size (ops.py:91-118): dw[c, t] = sum over
+// images and output positions of dy(p, q) * x(p*s + dh_t, q*s + dw_t), db[c] = sum of dy.
+// A workgroup owns four channels and every G-th (image, band) unit.  Per sub-tile it stages the
+// x window as planes (as fprop does) and the dy sub-tile as fp32 rows in LDS (zeros beyond the
+// image).  In sub-group k (channel k) a thread is (tap, part): it keeps the one running sum of
+// its tap over the part's share of the positions, four consecutive positions of a row at a time
+// (one 16-byte read of dy, broadcast to the taps, and four window elements).  The parts are
+// added at the end and the workgroup writes one partial per (channel, tap); db comes from the
+// threads that staged dy.
+template <typename T>
+constexpr size_t tile_wgrad_lds_bytes() {
+    return (size_t)kSliceCh * kTilePlaneElems * sizeof(T) + (size_t)kSliceCh * kTileOutputs * 4 + 64;
+}
+
+// Groups of (image, band) units: a multiple of 8 (unit u runs on XCD u % 8), about 8192
+// workgroups at most.
+inline int tile_wgrad_groups(const ConvDims &d, int *band_rows, int *nbands) {
+    const int nslices = (d.C + kSliceCh - 1) / kSliceCh;
+    *band_rows = tile_band_rows(d.N, d.P, nslices);
+    *nbands = (d.P + *band_rows - 1) / *band_rows;
+    const long units = ((long)d.N * *nbands + 7) / 8 * 8;
+    const long cap = (8192 / nslices + 7) / 8 * 8;
+    return (int)(units < cap ? units : cap);
+}
+
+template <typename T, class Src>
+__global__ __launch_bounds__(kTileThreads) __attribute__((amdgpu_waves_per_eu(4, 4))) void tile_wgrad_kernel(
+    typename Src::Params spx, typename Src::Params spy, const int8_t *__restrict__ dhdw,
+    float *__restrict__ part, ConvDims d, int nbands, int band_rows, int G, int slots_log2) {
+    extern __shared__ float lds_f[];
+    T *planes = reinterpret_cast<T *>(lds_f);
+    float *ldy = reinterpret_cast<float *>(planes + kSliceCh * kTilePlaneElems);  // [ch][th * tw]
+    int *halo = reinterpret_cast<int *>(ldy + kSliceCh * kTileOutputs);          // [ch][2]
+
+    const int nslices = (d.C + kSliceCh - 1) / kSliceCh;
+    const int g = blockIdx.x % 8 + 8 * (blockIdx.x / 8 / nslices);
+    const int slice = blockIdx.x / 8 % nslices;
+    const int c0 = slice * kSliceCh;
+    const int sub = __builtin_amdgcn_readfirstlane(threadIdx.x / kTileSub);
+    const unsigned stid = threadIdx.x % kTileSub;
+    const int c = min(c0 + sub, d.C - 1);
+    const int s_ = d.stride, K = d.K;
+    const int slots = 1 << slots_log2, parts = kTileSub >> slots_log2;
+    const int ts = stid & (slots - 1), prt = stid >> slots_log2;
+
+    const int8_t *mytaps = dhdw + (size_t)c * K * 2;
+    int hh = 0, hw = 0;
+    for (int s = 0; s < K; s++) {
+        hh = max(hh, abs((int)mytaps[2 * s]));
+        hw = max(hw, abs((int)mytaps[2 * s + 1]));
+    }
+    if (stid == 0) halo[sub * 2] = hh, halo[sub * 2 + 1] = hw;
+    __syncthreads();
+    hh = max(max(halo[0], halo[2]), max(halo[4], halo[6]));
+    hw = max(max(halo[1], halo[3]), max(halo[5], halo[7]));
+    hh = __builtin_amdgcn_readfirstlane(hh);
+    hw = __builtin_amdgcn_readfirstlane(hw);
+    const int rstep = hh == 0 ? s_ : 1, cstep = hw == 0 ? s_ : 1;
+    const int srow = s_ / rstep, scol = s_ / cstep;
+    // this thread's tap, in plane rows and columns (spare slots repeat tap 0 and are dropped)
+    const int my_dh = ts < K ? (int)mytaps[2 * ts] / rstep : 0;
+    const int my_dw = ts < K ? (int)mytaps[2 * ts + 1] / cstep : 0;
+
+    const T *plane = planes + sub * kTilePlaneElems;
+    const float *mydy = ldy + sub * kTileOutputs;
+    constexpr int PRE = kTilePlaneElems / kTileThreads, PREY = kTileOutputs / kTileThreads;
+    typename Src::Payload pre[PRE], prey[PREY];
+    Src srcx, srcy;
+    ConvDims dyd = d;  // dy as a source tensor: P x Q
+    dyd.H = d.P, dyd.W = d.Q;
+    float acc = 0.f, dsum[kSliceCh] = {0.f, 0.f, 0.f, 0.f};
+    const int Qe = max((d.Q + 3) & ~3, 8);  // sub-tile widths are multiples of 4
+
+    for (int unit = g; unit < d.N * nbands; unit += G) {
+        const int n = unit / nbands, band = unit - n * nbands;
+        const int p_lo = band * band_rows, p_hi = min(d.P, p_lo + band_rows);
+        int th, tw;
+        choose_tile(p_hi - p_lo, Qe, srow, scol, hh, hw, th, tw);
+        const int ih = (th - 1) * srow + 1 + 2 * hh;
+        const int iw = (tw - 1) * scol + 1 + 2 * hw;
+        const int iwp = iw | 1;
+        const int tw4 = tw >> 2;
+        const unsigned m_iw = div_magic(iw), m_tw = div_magic(tw), m_tw4 = div_magic(tw4);
+        const unsigned nwin = ih * iw, nout = th * tw, nquads = th * tw4;
+        const T *tapped = plane + (my_dh + hh) * iwp + my_dw + hw;
+        srcx.init(spx, n, c0, d);
+        srcy.init(spy, n, c0, dyd);
+
+        auto window_pixel = [&](int pt, int qt, unsigned v, unsigned &pixel) {
+            const unsigned i = fast_div(v, m_iw), j = v - i * iw;
+            const unsigned r = (unsigned)(pt * s_ - hh + (int)i * rstep);
+            const unsigned q = (unsigned)(qt * s_ - hw + (int)j * cstep);
+            pixel = r * d.W + q;
+            return v < nwin && r < (unsigned)d.H && q < (unsigned)d.W;
+        };
+        auto dy_pixel = [&](int pt, int qt, unsigned o, unsigned &pixel) {
+            const unsigned pl = fast_div(o, m_tw), ql = o - pl * tw;
+            const unsigned p = pt + pl, q = qt + ql;
+            pixel = p * d.Q + q;
+            return o < nout && p < (unsigned)p_hi && q < (unsigned)d.Q;
+        };
+        auto load_tiles = [&](int pt, int qt) {
+#pragma unroll
+            for (int u = 0; u < PRE; u++) {
+                if (u * kTileThreads >= (int)nwin) break;
+                unsigned v = u * kTileThreads + threadIdx.x;
+                asm volatile("" : "+v"(v));
+                unsigned pixel;
+                const bool inside = window_pixel(pt, qt, v, pixel);
+                srcx.load(pre[u], inside, pixel);
+            }
+#pragma unroll
+            for (int u = 0; u < PREY; u++) {
+                if (u * kTileThreads >= (int)nout) break;
+                unsigned o = u * kTileThreads + threadIdx.x;
+                asm volatile("" : "+v"(o));
+                unsigned pixel;
+                const bool inside = dy_pixel(pt, qt, o, pixel);
+                srcy.load(prey[u], inside, pixel);
+            }
+        };
+        load_tiles(p_lo, 0);
+        for (int pt = p_lo; pt < p_hi; pt += th) {
+            for (int qt = 0; qt < d.Q; qt += tw) {
+#pragma unroll
+                for (int u = 0; u < PRE; u++) {
+                    if (u * kTileThreads >= (int)nwin) break;
+                    unsigned v = u * kTileThreads + threadIdx.x;
+                    asm volatile("" : "+v"(v));
+                    if (v < nwin) {
+                        const unsigned i = fast_div(v, m_iw), j = v - i * iw;
+                        const unsigned at = i * iwp + j;
+                        unsigned pixel;
+                        const bool inside = window_pixel(pt, qt, v, pixel);
+#pragma unroll
+                        for (int ch = 0; ch < kSliceCh; ch++)
+                            planes[ch * kTilePlaneElems + at] = srcx.elem(pre[u], ch, inside);
+                    }
+                }
+#pragma unroll
+                for (int u = 0; u < PREY; u++) {
+                    if (u * kTileThreads >= (int)nout) break;
+                    const unsigned o = u * kTileThreads + threadIdx.x;
+                    if (o < nout) {
+#pragma unroll
+                        for (int ch = 0; ch < kSliceCh; ch++) {
+                            // (positions outside the image were loaded as zeros)
+                            const float v = to_float(srcy.elem(prey[u], ch, true));
+                            ldy[ch * kTileOutputs + o] = v;
+                            dsum[ch] += v;
+                        }
+                    }
+                }
+                __syncthreads();
+                if (qt + tw < d.Q)
+                    load_tiles(pt, qt + tw);
+                else if (pt + th < p_hi)
+                    load_tiles(pt + th, 0);
+#pragma unroll 2
+                for (unsigned qd = prt; qd < nquads; qd += parts) {
+                    const unsigned pl = fast_div(qd, m_tw4), qc = qd - pl * tw4;
+                    const float4 gy = *reinterpret_cast<const float4 *>(mydy + pl * tw + 4 * qc);
+                    const T *a = tapped + pl * srow * iwp + 4 * qc * scol;
+                    acc = __builtin_fmaf(gy.x, to_float(a[0]), acc);
+                    acc = __builtin_fmaf(gy.y, to_float(a[scol]), acc);
+                    acc = __builtin_fmaf(gy.z, to_float(a[2 * scol]), acc);
+                    acc = __builtin_fmaf(gy.w, to_float(a[3 * scol]), acc);
+                }
+                __syncthreads();
+            }
+        }
+    }
+
+    // parts -> one sum per (channel, tap); the dy sums of all threads -> one per channel
+    float *red = ldy;                       // [ch][128]
+    float *redb = ldy + kTileThreads;       // [wave][ch]
+    red[threadIdx.x] = acc;
+#pragma unroll
+    for (int ch = 0; ch < kSliceCh; ch++) {
+        float v = dsum[ch];
+#pragma unroll
+        for (int m = 32; m >= 1; m >>= 1) v += __shfl_xor(v, m, 64);
+        if (threadIdx.x % 64 == 0) redb[(threadIdx.x / 64) * kSliceCh + ch] = v;
+    }
+    __syncthreads();
+    if (c0 + sub >= d.C) return;
+    const size_t row = (size_t)c * (K + 1);
+    if (prt == 0 && ts < K) {
+        float total = 0.f;
+        for (int j = 0; j < parts; j++) total += red[sub * kTileSub + ts + (j << slots_log2)];
+        part[(row + ts) * G + g] = total;
+    }
+    if (stid == 0) {
+        float total = 0.f;
+        for (int wv = 0; wv < kTileThreads / 64; wv++) total += redb[wv * kSliceCh + sub];
+        part[(row + K) * G + g] = total;
+    }
+}
+
+// partial sums part[(c * (K + 1) + t) * G + g], t = K for db; returns G through `groups`
+template <typename T, class Src>
+int launch_tile_wgrad_src(const void *x, const void *dy, const void *taps, float *part, int *groups,
+                          const ConvDims &d, hipStream_t st) {
+    const size_t lds = tile_wgrad_lds_bytes<T>();
+    static const bool once = [&] {
+        allow_large_lds(tile_wgrad_kernel<T, Src>, lds);
+        return true;
+    }();
+    (void)once;
+    int band_rows, nbands;
+    const int G = tile_wgrad_groups(d, &band_rows, &nbands);
+    *groups = G;
+    const int nslices = (d.C + kSliceCh - 1) / kSliceCh;
+    int slots_log2 = 0;
+    while ((1 << slots_log2) < d.K) slots_log2++;
+    tile_wgrad_kernel<T, Src><<<dim3((unsigned)(G * nslices)), dim3(kTileThreads), lds, st>>>(
+        {(const T *)x}, {(const T *)dy}, taps_dhdw(taps), part, d, nbands, band_rows, G, slots_log2);
+    const hipError_t e = hipGetLastError();
+    return e == hipSuccess ? 0 : (int)e;
+}
+
+template <typename T>
+int launch_tile_wgrad(const void *x, const void *dy, const void *taps, float *part, int *groups,
+                      const ConvDims &d, bool nchw, hipStream_t st) {
+    return nchw ? launch_tile_wgrad_src<T, PlaneSource<T>>(x, dy, taps, part, groups, d, st)
+                : launch_tile_wgrad_src<T, SliceSource<T>>(x, dy, taps, part, groups, d, st);
 }
 
 }  // namespace dwo
