@@ -97,6 +97,18 @@ def test_stage_shapes_k15(oracle, C, HW, nhwc, dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("nhwc", [False, True], ids=["nchw", "nhwc"])
+@pytest.mark.parametrize("C,HW", [(48, 56), (64, 28), (96, 14), (128, 7)])
+def test_stage_shapes_reversed_orientations(oracle, C, HW, nhwc, dtype):
+    """Angles of the layers turned by 90 degrees (models/convnext.py:159-160): half of them lie
+    in [180, 270) degrees, where the taps are a canonical pattern in reverse order."""
+    theta = (canonical_theta(C) + np.float32(math.pi / 2)).astype(np.float32)
+    _case(oracle, 3, C, HW, HW, 31, 1, dtype, nhwc, theta, seed=C + HW + 90)
+    theta = (canonical_theta(C) + np.float32(math.pi)).astype(np.float32)
+    _case(oracle, 2, C, HW, HW, 31, 1, dtype, nhwc, theta, seed=C + HW + 180)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
 @pytest.mark.parametrize("C,HW", [(40, 56), (40, 28), (72, 14), (100, 7)])
 def test_stage_shapes_mixed_angles(oracle, C, HW, dtype):
     """Stage plane extents with arbitrary angles mixed among canonical ones (a workgroup picks
