@@ -145,6 +145,9 @@ int try_nhwc_plane_wgrad(const void *x, const void *dy, const void *taps, float 
 // below 2 GB (32-bit offsets inside one)
 bool tile_covers(const ConvDims &d, int layout, size_t esize) {
     if ((size_t)d.H * d.W * d.C * esize >= 0x80000000ull) return false;
+    // the smallest sub-tile (1 x 8 outputs) of the widest possible taps must fit a channel plane
+    const int plane = esize == 2 ? tile_plane_elems<bf16_t>() : tile_plane_elems<float>();
+    if (d.K * ((7 * d.stride + d.K) | 1) > plane) return false;
     return layout == DWO_NCHW || d.C % kSliceCh == 0;
 }
 

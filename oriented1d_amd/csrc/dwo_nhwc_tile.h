@@ -23,15 +23,18 @@ namespace dwo {
 
 constexpr int kTileThreads = 512;                          // four sub-groups of two waves
 constexpr int kTileSub = kTileThreads / kSliceCh;          // threads per channel
-constexpr int kTilePlaneElems = 7680;                      // LDS elements per channel plane (two
-                                                           // workgroups of 16-bit planes per CU)
+// LDS elements per channel plane: two workgroups per CU for every element type
+template <typename T>
+constexpr int tile_plane_elems() {
+    return sizeof(T) == 2 ? 7680 : 3584;
+}
 constexpr int kTileOutputs = 1024;                         // most outputs per sub-tile
 constexpr int kTileBandRows = 32;                          // most output rows per workgroup
 
 // planes, fp32 results, per-channel tap table (offset, weight) and tap extents
 template <typename T>
 constexpr size_t nhwc_tile_lds_bytes() {
-    return (size_t)kSliceCh * kTilePlaneElems * sizeof(T) + (size_t)kSliceCh * kTileOutputs * 4 +
+    return (size_t)kSliceCh * tile_plane_elems<T>() * sizeof(T) + (size_t)kSliceCh * kTileOutputs * 4 +
            (size_t)kSliceCh * DWO_MAX_K * 8 + 64;
 }
 
@@ -221,7 +224,7 @@ __device__ __forceinline__ void tile_flush(const float *lout, int stride, T *yn,
 // cross products.  Widths: the full width `wfull` or a power of two from 8 to 128; widths of at
 // least 2, also for a one-column plane: the index arithmetic divides by them.
 __device__ __forceinline__ void choose_tile(int RH, int wfull, int srow, int scol, int hh, int hw,
-                                            int &th, int &tw) {
+                                            int plane_elems, int &th, int &tw) {
     th = 1, tw = min(wfull, 8);
     int best_num = 0x7fffffff / kTileOutputs, best_den = 1;
     for (int a = RH; a >= 1; a = (a + 1) / 2) {
@@ -229,7 +232,7 @@ __device__ __forceinline__ void choose_tile(int RH, int wfull, int srow, int sco
             const int b = k == 0 ? wfull : (256 >> k);
             if (b > wfull || a * b > kTileOutputs) continue;
             const int ih = (a - 1) * srow + 1 + 2 * hh, iw = ((b - 1) * scol + 1 + 2 * hw) | 1;
-            if (ih * iw > kTilePlaneElems) continue;
+            if (ih * iw > plane_elems) continue;
             const int num = ih * iw + 1536, den = a * b;
             if (num * best_den < best_num * den) best_num = num, best_den = den, th = a, tw = b;
         }
@@ -251,7 +254,7 @@ __global__ __launch_bounds__(kTileThreads) __attribute__((amdgpu_waves_per_eu(4,
     int flip) {
     extern __shared__ float lds_f[];
     T *planes = reinterpret_cast<T *>(lds_f);
-    float *lout = reinterpret_cast<float *>(planes + kSliceCh * kTilePlaneElems);
+    float *lout = reinterpret_cast<float *>(planes + kSliceCh * tile_plane_elems<T>());
     int2 *tapt = reinterpret_cast<int2 *>(lout + kSliceCh * kTileOutputs);  // [ch][K] (offset, weight)
     int *halo = reinterpret_cast<int *>(tapt + kSliceCh * DWO_MAX_K);       // [ch][2]
 
@@ -296,7 +299,7 @@ __global__ __launch_bounds__(kTileThreads) __attribute__((amdgpu_waves_per_eu(4,
     const int RH = p_hi - p_lo;
     const int Qe = max(d.Q, 2);
     int th, tw;
-    choose_tile(RH, Qe, srow, scol, hh, hw, th, tw);
+    choose_tile(RH, Qe, srow, scol, hh, hw, tile_plane_elems<T>(), th, tw);
     const int ih = (th - 1) * srow + 1 + 2 * hh;
     const int iw = (tw - 1) * scol + 1 + 2 * hw;
     const int iwp = iw | 1;
@@ -308,11 +311,11 @@ __global__ __launch_bounds__(kTileThreads) __attribute__((amdgpu_waves_per_eu(4,
                                 __float_as_int(wt[(size_t)c * K + (flip ? K - 1 - (int)stid : (int)stid)]));
 
     T *yn = Src::kNchw ? y + ((size_t)n * d.C + c0) * d.P * d.Q : y + (size_t)n * d.P * d.Q * d.C + c0;
-    const T *plane = planes + sub * kTilePlaneElems;
+    const T *plane = planes + sub * tile_plane_elems<T>();
     const unsigned nwin = ih * iw, nout = th * tw;
 
     // window of sub-tile (pt, qt) -> registers: rows pt*s - hh .., columns qt*s - hw ..
-    constexpr int PRE = kTilePlaneElems / kTileThreads;  // pixels per thread, at most
+    constexpr int PRE = tile_plane_elems<T>() / kTileThreads;  // pixels per thread, at most
     typename Src::Payload pre[PRE];
     Src source;
     source.init(sp, n, c0, d);
@@ -349,7 +352,7 @@ __global__ __launch_bounds__(kTileThreads) __attribute__((amdgpu_waves_per_eu(4,
                     const bool inside = window_pixel(pt, qt, v, pixel);
 #pragma unroll
                     for (int ch = 0; ch < kSliceCh; ch++)
-                        planes[ch * kTilePlaneElems + at] = source.elem(pre[u], ch, inside);
+                        planes[ch * tile_plane_elems<T>() + at] = source.elem(pre[u], ch, inside);
                 }
             }
             __syncthreads();
@@ -441,13 +444,17 @@ int launch_nhwc_tile_pointwise_fprop(const void *x, const float *pw_w, const flo
 // sub-tile it stages the dy window as one plane per channel in LDS, lets sub-group k evaluate
 // channel k class after class (its tap table is sorted by class), places the sums at their dx
 // positions in LDS and writes the sub-tile out in raster order.
-constexpr int kDgradPlaneElems = 4096;  // LDS elements per channel plane (dy window)
+// LDS elements per channel plane (dy window): two workgroups per CU for every element type
+template <typename T>
+constexpr int dgrad_plane_elems() {
+    return sizeof(T) == 2 ? 4096 : 2048;
+}
 constexpr int kDgradOutputs = 2048;     // most dx pixels per sub-tile
 constexpr int kDgradClasses = 16;       // residue classes at stride 4
 
 template <typename T>
 constexpr size_t tile_dgrad_lds_bytes() {
-    return (size_t)kSliceCh * kDgradPlaneElems * sizeof(T) + (size_t)kSliceCh * kDgradOutputs * 4 +
+    return (size_t)kSliceCh * dgrad_plane_elems<T>() * sizeof(T) + (size_t)kSliceCh * kDgradOutputs * 4 +
            (size_t)kSliceCh * DWO_MAX_K * 8 + (size_t)kSliceCh * (kDgradClasses + 1) * 4 + 64;
 }
 
@@ -457,7 +464,7 @@ __global__ __launch_bounds__(kTileThreads) __attribute__((amdgpu_waves_per_eu(4,
     T *__restrict__ dx, ConvDims d, int nbands, int band_rows) {
     extern __shared__ float lds_f[];
     T *planes = reinterpret_cast<T *>(lds_f);
-    float *lout = reinterpret_cast<float *>(planes + kSliceCh * kDgradPlaneElems);
+    float *lout = reinterpret_cast<float *>(planes + kSliceCh * dgrad_plane_elems<T>());
     int2 *tapt = reinterpret_cast<int2 *>(lout + kSliceCh * kDgradOutputs);  // [ch][K], by class
     int *cstart = reinterpret_cast<int *>(tapt + kSliceCh * DWO_MAX_K);     // [ch][classes + 1]
     int *halo = cstart + kSliceCh * (kDgradClasses + 1);                    // [ch][2]
@@ -506,7 +513,7 @@ __global__ __launch_bounds__(kTileThreads) __attribute__((amdgpu_waves_per_eu(4,
                 const int b = k < 0 ? We : (256 >> k);  // full width, 256, 128, 64, 32, 16, 8
                 if (b > We || a * b > kDgradOutputs) continue;
                 const int ih = (a >> sh) + 2 * hh, iw = ((b >> sh) + 2 * hw) | 1;
-                if (ih * iw > kDgradPlaneElems) continue;
+                if (ih * iw > dgrad_plane_elems<T>()) continue;
                 const float cost = (float)(ih * iw + 1536) / (float)(a * b);
                 if (cost < best) best = cost, th = a, tw = b;
             }
@@ -538,10 +545,10 @@ __global__ __launch_bounds__(kTileThreads) __attribute__((amdgpu_waves_per_eu(4,
     }
 
     T *dxn = Src::kNchw ? dx + ((size_t)n * d.C + c0) * d.H * d.W : dx + (size_t)n * d.H * d.W * d.C + c0;
-    const T *plane = planes + sub * kDgradPlaneElems;
+    const T *plane = planes + sub * dgrad_plane_elems<T>();
     float *myout = lout + sub * kDgradOutputs;
 
-    constexpr int PRE = kDgradPlaneElems / kTileThreads;
+    constexpr int PRE = dgrad_plane_elems<T>() / kTileThreads;
     typename Src::Payload pre[PRE];
     Src source;
     ConvDims ds = d;  // the source tensor is dy: P x Q
@@ -606,7 +613,7 @@ __global__ __launch_bounds__(kTileThreads) __attribute__((amdgpu_waves_per_eu(4,
                     const bool inside = window_pixel(ht, wt_, v, pixel);
 #pragma unroll
                     for (int ch = 0; ch < kSliceCh; ch++)
-                        planes[ch * kDgradPlaneElems + at] = source.elem(pre[u], ch, inside);
+                        planes[ch * dgrad_plane_elems<T>() + at] = source.elem(pre[u], ch, inside);
                 }
             }
             __syncthreads();
@@ -674,7 +681,7 @@ int launch_tile_dgrad_strided(const void *dy, const float *w, const void *taps, 
 // threads that staged dy.
 template <typename T>
 constexpr size_t tile_wgrad_lds_bytes() {
-    return (size_t)kSliceCh * kTilePlaneElems * sizeof(T) + (size_t)kSliceCh * kTileOutputs * 4 + 64;
+    return (size_t)kSliceCh * tile_plane_elems<T>() * sizeof(T) + (size_t)kSliceCh * kTileOutputs * 4 + 64;
 }
 
 // Groups of (image, band) units: a multiple of 8 (unit u runs on XCD u % 8), about 8192
@@ -694,7 +701,7 @@ __global__ __launch_bounds__(kTileThreads) __attribute__((amdgpu_waves_per_eu(4,
     float *__restrict__ part, ConvDims d, int nbands, int band_rows, int G, int slots_log2) {
     extern __shared__ float lds_f[];
     T *planes = reinterpret_cast<T *>(lds_f);
-    float *ldy = reinterpret_cast<float *>(planes + kSliceCh * kTilePlaneElems);  // [ch][th * tw]
+    float *ldy = reinterpret_cast<float *>(planes + kSliceCh * tile_plane_elems<T>());  // [ch][th * tw]
     int *halo = reinterpret_cast<int *>(ldy + kSliceCh * kTileOutputs);          // [ch][2]
 
     const int nslices = (d.C + kSliceCh - 1) / kSliceCh;
@@ -726,9 +733,9 @@ __global__ __launch_bounds__(kTileThreads) __attribute__((amdgpu_waves_per_eu(4,
     const int my_dh = ts < K ? (int)mytaps[2 * ts] / rstep : 0;
     const int my_dw = ts < K ? (int)mytaps[2 * ts + 1] / cstep : 0;
 
-    const T *plane = planes + sub * kTilePlaneElems;
+    const T *plane = planes + sub * tile_plane_elems<T>();
     const float *mydy = ldy + sub * kTileOutputs;
-    constexpr int PRE = kTilePlaneElems / kTileThreads, PREY = kTileOutputs / kTileThreads;
+    constexpr int PRE = tile_plane_elems<T>() / kTileThreads, PREY = kTileOutputs / kTileThreads;
     typename Src::Payload pre[PRE], prey[PREY];
     Src srcx, srcy;
     ConvDims dyd = d;  // dy as a source tensor: P x Q
@@ -740,7 +747,7 @@ __global__ __launch_bounds__(kTileThreads) __attribute__((amdgpu_waves_per_eu(4,
         const int n = unit / nbands, band = unit - n * nbands;
         const int p_lo = band * band_rows, p_hi = min(d.P, p_lo + band_rows);
         int th, tw;
-        choose_tile(p_hi - p_lo, Qe, srow, scol, hh, hw, th, tw);
+        choose_tile(p_hi - p_lo, Qe, srow, scol, hh, hw, tile_plane_elems<T>(), th, tw);
         const int ih = (th - 1) * srow + 1 + 2 * hh;
         const int iw = (tw - 1) * scol + 1 + 2 * hw;
         const int iwp = iw | 1;
@@ -799,7 +806,7 @@ __global__ __launch_bounds__(kTileThreads) __attribute__((amdgpu_waves_per_eu(4,
                         const bool inside = window_pixel(pt, qt, v, pixel);
 #pragma unroll
                         for (int ch = 0; ch < kSliceCh; ch++)
-                            planes[ch * kTilePlaneElems + at] = srcx.elem(pre[u], ch, inside);
+                            planes[ch * tile_plane_elems<T>() + at] = srcx.elem(pre[u], ch, inside);
                     }
                 }
 #pragma unroll
