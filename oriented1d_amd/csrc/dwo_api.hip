@@ -337,7 +337,7 @@ const char *dwo_status_string(int status) {
 
 size_t dwo_taps_bytes(int C, int K) {
     if (C < 1 || K < 1 || K > DWO_MAX_K || (K & 1) == 0) return 0;
-    return kTapsHeaderBytes + taps_dhdw_bytes(C, K) + 2 * taps_class_bytes(C);
+    return kTapsHeaderBytes + taps_dhdw_bytes(C, K) + 2 * taps_class_bytes(C) + taps_extent_bytes(C);
 }
 
 int dwo_build_taps(const float *theta_host, int C, int K, void *taps_host) {
@@ -394,6 +394,14 @@ int dwo_build_taps(const float *theta_host, int C, int K, void *taps_host) {
             if (c < C) order[placed++] = c;
         }
     }
+    hdr[7] = hdr[6] + (int32_t)taps_class_bytes(C);
+    int8_t *extent = (int8_t *)taps_host + hdr[7];
+    for (int c = 0; c < C; c++)
+        for (int s = 0; s < K; s++)
+            for (int k = 0; k < 2; k++) {
+                const int a = abs((int)dhdw[((size_t)c * K + s) * 2 + k]);
+                if (a > extent[2 * c + k]) extent[2 * c + k] = (int8_t)a;
+            }
     return DWO_OK;
 }
 

@@ -10,7 +10,7 @@ namespace dwo {
 
 // ---------------------------------------------------------------------------------------------
 // Tap blob (private layout).  Built on the host by dwo_build_taps, copied verbatim to the device.
-//   int32 header[8] : magic, version, C, K, off_dhdw, off_class, off_order, 0
+//   int32 header[8] : magic, version, C, K, off_dhdw, off_class, off_order, off_extent
 //   int8  dhdw[C][K][2]        (dh, dw) of every tap, padded to 16 bytes
 //   int32 cls[C]               canonical orientation id 0..7 of the channel's tap pattern
 //                              (k * 22.5 degrees), or -1 when the pattern is not canonical;
@@ -20,9 +20,10 @@ namespace dwo {
 //                              workgroups take their channel from it, so that whatever way the
 //                              angles are laid out over the channels, neighbouring workgroup
 //                              ids (hence every XCD and CU) get a mix of orientations
+//   int8  extent[C][2]         (max |dh|, max |dw|) over the channel's taps, padded to 16 bytes
 // ---------------------------------------------------------------------------------------------
 constexpr int32_t kTapsMagic = 0x44574f31;  // "DWO1"
-constexpr int32_t kTapsVersion = 3;
+constexpr int32_t kTapsVersion = 4;
 constexpr int kTapsHeaderInts = 8;
 constexpr int kTapsHeaderBytes = kTapsHeaderInts * 4;
 
@@ -43,6 +44,13 @@ __host__ __device__ inline bool class_reversed(int cls) { return cls >= 8; }
 __host__ __device__ inline const int32_t *taps_class(const void *blob, int C, int K) {
     return reinterpret_cast<const int32_t *>(reinterpret_cast<const int8_t *>(blob) +
                                              kTapsHeaderBytes + taps_dhdw_bytes(C, K));
+}
+__host__ __device__ inline size_t taps_extent_bytes(int C) {
+    return ((size_t)C * 2 + 15) & ~(size_t)15;
+}
+__host__ __device__ inline const int8_t *taps_extent(const void *blob, int C, int K) {
+    return reinterpret_cast<const int8_t *>(blob) + kTapsHeaderBytes + taps_dhdw_bytes(C, K) +
+           2 * taps_class_bytes(C);
 }
 __host__ __device__ inline const int32_t *taps_order(const void *blob, int C, int K) {
     return reinterpret_cast<const int32_t *>(reinterpret_cast<const int8_t *>(blob) +

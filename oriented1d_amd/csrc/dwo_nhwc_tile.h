@@ -29,13 +29,15 @@ constexpr int tile_plane_elems() {
     return sizeof(T) == 2 ? 7680 : 3584;
 }
 constexpr int kTileOutputs = 1024;                         // most outputs per sub-tile
+constexpr int kTileTapSlots = (DWO_MAX_K + 3) / 4 * 4 + 4;  // tap table: whole groups of four taps
+                                                           // plus one group read ahead
 constexpr int kTileBandRows = 32;                          // most output rows per workgroup
 
 // planes, fp32 results, per-channel tap table (offset, weight) and tap extents
 template <typename T>
 constexpr size_t nhwc_tile_lds_bytes() {
     return (size_t)kSliceCh * tile_plane_elems<T>() * sizeof(T) + (size_t)kSliceCh * kTileOutputs * 4 +
-           (size_t)kSliceCh * DWO_MAX_K * 8 + 64;
+           (size_t)kSliceCh * kTileTapSlots * 8 + 64;
 }
 
 // One pixel slice at byte offset `off` of a raw buffer descriptor (zeros when off lies outside).
@@ -185,9 +187,7 @@ struct PointwiseSource {
 
 // floor(n / d) for n < 2^16 and 2 <= d < 2^16, with m = ceil(2^32 / d)
 __device__ __forceinline__ unsigned fast_div(unsigned n, unsigned m) { return __umulhi(n, m); }
-__device__ __forceinline__ unsigned div_magic(unsigned d) {
-    return (unsigned)((0x100000000ull + d - 1) / d);
-}
+__device__ __forceinline__ unsigned div_magic(unsigned d) { return 0xffffffffu / d + 1; }
 
 // Results of a th x tw sub-tile at (pt, qt), one fp32 plane of `stride` floats per channel in
 // `lout`, to the image at `yn` (rows below p_hi, columns below Q): NCHW as rows of each channel
@@ -216,6 +216,21 @@ __device__ __forceinline__ void tile_flush(const float *lout, int stride, T *yn,
             }
         }
     }
+}
+
+// Largest |dh| and |dw| over the taps of channels c0 .. c0+3 (uniform), from the tap blob's
+// per-channel extents.
+__device__ __forceinline__ void slice_extent(const int8_t *__restrict__ extent, int c0, int C, int &hh,
+                                             int &hw) {
+    hh = 0, hw = 0;
+#pragma unroll
+    for (int ch = 0; ch < kSliceCh; ch++) {
+        const int c = min(c0 + ch, C - 1);
+        hh = max(hh, (int)extent[2 * c]);
+        hw = max(hw, (int)extent[2 * c + 1]);
+    }
+    hh = __builtin_amdgcn_readfirstlane(hh);
+    hw = __builtin_amdgcn_readfirstlane(hw);
 }
 
 // Sub-tile shape for a band of RH output rows: th rows x tw columns of outputs with a window
@@ -250,13 +265,12 @@ inline int tile_band_rows(int N, int rows, int nslices) {
 template <typename T, class Src>
 __global__ __launch_bounds__(kTileThreads) __attribute__((amdgpu_waves_per_eu(4, 4))) void nhwc_tile_fprop_kernel(
     typename Src::Params sp, const float *__restrict__ wt, const float *__restrict__ bias,
-    const int8_t *__restrict__ dhdw, T *__restrict__ y, ConvDims d, int nbands, int band_rows,
-    int flip) {
+    const int8_t *__restrict__ dhdw, const int8_t *__restrict__ extent, T *__restrict__ y, ConvDims d,
+    int nbands, int band_rows, int flip) {
     extern __shared__ float lds_f[];
     T *planes = reinterpret_cast<T *>(lds_f);
     float *lout = reinterpret_cast<float *>(planes + kSliceCh * tile_plane_elems<T>());
     int2 *tapt = reinterpret_cast<int2 *>(lout + kSliceCh * kTileOutputs);  // [ch][K] (offset, weight)
-    int *halo = reinterpret_cast<int *>(tapt + kSliceCh * DWO_MAX_K);       // [ch][2]
 
     // Unit (image, band) u runs on XCD u % 8: hardware deals consecutive workgroup ids to the
     // XCDs in turn, so the slices of one band (which share every cache line they touch, NHWC)
@@ -272,43 +286,44 @@ __global__ __launch_bounds__(kTileThreads) __attribute__((amdgpu_waves_per_eu(4,
     const int c = min(c0 + sub, d.C - 1);  // (a partial last group repeats its last channel)
     const int s_ = d.stride, K = d.K;
 
-    // tap extents of this sub-group's channel (uniform), then of the four channels together
+    // tap extents of the four channels together
     const int8_t *mytaps = dhdw + (size_t)c * K * 2;
-    int hh = 0, hw = 0;
-    for (int s = 0; s < K; s++) {
-        hh = max(hh, abs((int)mytaps[2 * s]));
-        hw = max(hw, abs((int)mytaps[2 * s + 1]));
-    }
-    if (stid == 0) halo[sub * 2] = hh, halo[sub * 2 + 1] = hw;
-    __syncthreads();
-    hh = max(max(halo[0], halo[2]), max(halo[4], halo[6]));
-    hw = max(max(halo[1], halo[3]), max(halo[5], halo[7]));
-    hh = __builtin_amdgcn_readfirstlane(hh);
-    hw = __builtin_amdgcn_readfirstlane(hw);
+    int hh, hw;
+    slice_extent(extent, c0, d.C, hh, hw);
     const float bv = bias != nullptr ? bias[c] : 0.f;
 
     // Window rows/columns step by the stride when no tap of the slice leaves its row/column
     // (0 and 90 degrees): the positions in between are never read.
     const int rstep = hh == 0 ? s_ : 1, cstep = hw == 0 ? s_ : 1;
-    const int srow = s_ / rstep, scol = s_ / cstep;  // plane rows/columns per output row/column
+    const int srow = hh == 0 ? 1 : s_, scol = hw == 0 ? 1 : s_;  // plane rows/columns per output row/column
 
     // sub-tile shape: th rows x tw columns of outputs; window ih x iw of inputs.  Cost per
     // output = window positions plus a fixed per-sub-tile charge (barriers, pipeline fill).
     // (widths of at least 2, also for a one-column plane: the index arithmetic divides by them)
     const int p_lo = band * band_rows, p_hi = min(d.P, p_lo + band_rows);
     const int RH = p_hi - p_lo;
-    const int Qe = max(d.Q, 2);
+    const int Qe = max((d.Q + 1) & ~1, 2);  // even widths: a thread evaluates pairs of columns
     int th, tw;
     choose_tile(RH, Qe, srow, scol, hh, hw, tile_plane_elems<T>(), th, tw);
     const int ih = (th - 1) * srow + 1 + 2 * hh;
     const int iw = (tw - 1) * scol + 1 + 2 * hw;
     const int iwp = iw | 1;
     const unsigned m_iw = div_magic(iw), m_tw = div_magic(tw);
-    // the channel's taps as (LDS element offset, weight) pairs, read back as broadcasts
-    int2 *mytab = tapt + sub * DWO_MAX_K;
-    if ((int)stid < K)
-        mytab[stid] = make_int2(((int)mytaps[2 * stid] / rstep) * iwp + (int)mytaps[2 * stid + 1] / cstep,
-                                __float_as_int(wt[(size_t)c * K + (flip ? K - 1 - (int)stid : (int)stid)]));
+    // the channel's taps as (LDS byte offset, weight) pairs, read back as broadcasts; padded with
+    // weightless taps to whole groups of four plus the group that is read ahead
+    int2 *mytab = tapt + sub * kTileTapSlots;
+    const int K4 = (K + 3) & ~3;
+    if ((int)stid < K4 + 4) {
+        int2 e = make_int2(0, 0);
+        if ((int)stid < K)
+            // (the steps exceed 1 only where every offset of the slice is 0: no division needed)
+            e = make_int2(((int)mytaps[2 * stid] * iwp + (int)mytaps[2 * stid + 1]) *
+                              (int)sizeof(T),
+                          __float_as_int(wt[(size_t)c * K + (flip ? K - 1 - (int)stid : (int)stid)]));
+        mytab[stid] = e;
+    }
+    const unsigned long long *mytab64 = reinterpret_cast<const unsigned long long *>(mytab);
+    const unsigned tw2 = tw >> 1, m_tw2 = div_magic(max(tw2, 2u)), npairs = th * tw2;
 
     T *yn = Src::kNchw ? y + ((size_t)n * d.C + c0) * d.P * d.Q : y + (size_t)n * d.P * d.Q * d.C + c0;
     const T *plane = planes + sub * tile_plane_elems<T>();
@@ -361,30 +376,61 @@ __global__ __launch_bounds__(kTileThreads) __attribute__((amdgpu_waves_per_eu(4,
                 load_window(pt, qt + tw);
             else if (pt + th < p_hi)
                 load_window(pt + th, 0);
-            // sub-group: one channel; a thread takes four outputs at a time so that each tap's
-            // (offset, weight) is fetched once for the four
-            for (unsigned o0 = stid; o0 < nout; o0 += 4 * kTileSub) {
-                const T *base[4];
-                float acc[4];
+            // sub-group: one channel; a thread takes two pairs of neighbouring outputs at a time:
+            // each tap's (offset, weight) is fetched once for the four, each pair shares one
+            // address, and the next four taps travel while these are used
+            auto eval = [&](auto sc) {
+                constexpr int SB = decltype(sc)::value * (int)sizeof(T);  // bytes between the pair
+                for (unsigned i0 = stid; i0 < npairs; i0 += 2 * kTileSub) {
+                    const char *base[2];
+                    unsigned at[2];
+                    float acc[4] = {bv, bv, bv, bv};
 #pragma unroll
-                for (int k = 0; k < 4; k++) {
-                    const unsigned o = min(o0 + k * kTileSub, nout - 1);
-                    const unsigned pl = fast_div(o, m_tw), ql = o - pl * tw;
-                    base[k] = plane + ((pl * srow + hh) * iwp + ql * scol + hw);
-                    acc[k] = bv;
+                    for (int k = 0; k < 2; k++) {
+                        const unsigned i = min(i0 + k * kTileSub, npairs - 1);
+                        const unsigned pl = tw2 == 1 ? i : fast_div(i, m_tw2), ql = 2 * (i - pl * tw2);
+                        base[k] = reinterpret_cast<const char *>(
+                            plane + ((pl * srow + hh) * iwp + ql * decltype(sc)::value + hw));
+                        at[k] = pl * tw + ql;
+                    }
+                    unsigned long long cur[4], nxt[4];
+#pragma unroll
+                    for (int j = 0; j < 4; j++) cur[j] = mytab64[j];
+                    for (int s = 0; s < K4; s += 4) {
+#pragma unroll
+                        for (int j = 0; j < 4; j++) nxt[j] = mytab64[s + 4 + j];
+                        T v[4][4];
+#pragma unroll
+                        for (int j = 0; j < 4; j++) {
+#pragma unroll
+                            for (int k = 0; k < 2; k++) {
+                                const char *a = base[k] + (int)cur[j];
+                                v[j][2 * k] = *reinterpret_cast<const T *>(a);
+                                v[j][2 * k + 1] = *reinterpret_cast<const T *>(a + SB);
+                            }
+                        }
+#pragma unroll
+                        for (int j = 0; j < 4; j++) {
+                            const float w = __int_as_float((int)(cur[j] >> 32));
+#pragma unroll
+                            for (int k = 0; k < 4; k++) acc[k] = __builtin_fmaf(to_float(v[j][k]), w, acc[k]);
+                        }
+#pragma unroll
+                        for (int j = 0; j < 4; j++) cur[j] = nxt[j];
+                    }
+#pragma unroll
+                    for (int k = 0; k < 2; k++)
+                        if (i0 + k * kTileSub < npairs)
+                            *reinterpret_cast<float2 *>(lout + sub * kTileOutputs + at[k]) =
+                                make_float2(acc[2 * k], acc[2 * k + 1]);
                 }
-#pragma unroll 4
-                for (int s = 0; s < K; s++) {
-                    const int2 t = mytab[s];
-                    const float w = __int_as_float(t.y);
-#pragma unroll
-                    for (int k = 0; k < 4; k++)
-                        acc[k] = __builtin_fmaf(to_float(base[k][t.x]), w, acc[k]);
-                }
-#pragma unroll
-                for (int k = 0; k < 4; k++)
-                    if (o0 + k * kTileSub < nout) lout[sub * kTileOutputs + o0 + k * kTileSub] = acc[k];
-            }
+            };
+            if (scol == 1)
+                eval(std::integral_constant<int, 1>{});
+            else if (scol == 2)
+                eval(std::integral_constant<int, 2>{});
+            else
+                eval(std::integral_constant<int, 4>{});
             __syncthreads();
             tile_flush<T, Src::kNchw>(lout, kTileOutputs, yn, nout, tw, m_tw, pt, qt, p_hi, d.P, d.Q, d.C,
                                       c0);
@@ -408,7 +454,7 @@ int launch_nhwc_tile(const typename Src::Params &sp, const float *w, const float
     const long grid = 8L * (((long)d.N * nbands + 7) / 8) * nslices;
     if (grid > 0x7fffffffL) return DWO_ERR_BAD_SHAPE;
     nhwc_tile_fprop_kernel<T, Src><<<dim3((unsigned)grid), dim3(kTileThreads), lds, st>>>(
-        sp, w, bias, taps_dhdw(taps), (T *)y, d, nbands, band_rows, flip);
+        sp, w, bias, taps_dhdw(taps), taps_extent(taps, d.C, d.K), (T *)y, d, nbands, band_rows, flip);
     const hipError_t e = hipGetLastError();
     return e == hipSuccess ? 0 : (int)e;
 }
@@ -455,19 +501,19 @@ constexpr int kDgradClasses = 16;       // residue classes at stride 4
 template <typename T>
 constexpr size_t tile_dgrad_lds_bytes() {
     return (size_t)kSliceCh * dgrad_plane_elems<T>() * sizeof(T) + (size_t)kSliceCh * kDgradOutputs * 4 +
-           (size_t)kSliceCh * DWO_MAX_K * 8 + (size_t)kSliceCh * (kDgradClasses + 1) * 4 + 64;
+           (size_t)kSliceCh * DWO_MAX_K * 12 + (size_t)kSliceCh * (kDgradClasses + 1) * 4 + 64;
 }
 
 template <typename T, class Src>
 __global__ __launch_bounds__(kTileThreads) __attribute__((amdgpu_waves_per_eu(4, 4))) void tile_dgrad_strided_kernel(
     typename Src::Params sp, const float *__restrict__ wt, const int8_t *__restrict__ dhdw,
-    T *__restrict__ dx, ConvDims d, int nbands, int band_rows) {
+    const int8_t *__restrict__ extent, T *__restrict__ dx, ConvDims d, int nbands, int band_rows) {
     extern __shared__ float lds_f[];
     T *planes = reinterpret_cast<T *>(lds_f);
     float *lout = reinterpret_cast<float *>(planes + kSliceCh * dgrad_plane_elems<T>());
     int2 *tapt = reinterpret_cast<int2 *>(lout + kSliceCh * kDgradOutputs);  // [ch][K], by class
     int *cstart = reinterpret_cast<int *>(tapt + kSliceCh * DWO_MAX_K);     // [ch][classes + 1]
-    int *halo = cstart + kSliceCh * (kDgradClasses + 1);                    // [ch][2]
+    int *halo = cstart + kSliceCh * (kDgradClasses + 1);                    // [ch][K] taps
 
     const int nslices = (d.C + kSliceCh - 1) / kSliceCh;
     const int unit = blockIdx.x % 8 + 8 * (blockIdx.x / 8 / nslices);
@@ -480,26 +526,22 @@ __global__ __launch_bounds__(kTileThreads) __attribute__((amdgpu_waves_per_eu(4,
     const int c = min(c0 + sub, d.C - 1);
     const int s_ = d.stride, sh = d.shift, K = d.K, ncls = s_ * s_;
 
-    // tap t: residue class and offset in dy
+    // the channel's taps into LDS (each is looked at K times below); tap t: residue class and
+    // offset in dy
     const int8_t *mytaps = dhdw + (size_t)c * K * 2;
+    int *ltap = halo + sub * DWO_MAX_K;
+    if ((int)stid < K) ltap[stid] = ((int)mytaps[2 * stid] << 16) | ((int)mytaps[2 * stid + 1] & 0xffff);
     auto tap_class = [&](int t, int &eh, int &ew) {
-        const int dh = mytaps[2 * t], dw = mytaps[2 * t + 1];
+        const int packed = ltap[t];
+        const int dh = packed >> 16, dw = (int)(short)packed;
         eh = -(dh >> sh), ew = -(dw >> sh);  // (arithmetic shifts: floor)
         return (dh & (s_ - 1)) * s_ + (dw & (s_ - 1));
     };
-    int hh = 0, hw = 0;
-    for (int t = 0; t < K; t++) {
-        int eh, ew;
-        tap_class(t, eh, ew);
-        hh = max(hh, abs(eh));
-        hw = max(hw, abs(ew));
-    }
-    if (stid == 0) halo[sub * 2] = hh, halo[sub * 2 + 1] = hw;
+    // extents in dy: the taps are symmetric about the centre, so |floor(-e / s)| = ceil(e / s)
+    int hh, hw;
+    slice_extent(extent, c0, d.C, hh, hw);
+    hh = (hh + s_ - 1) >> sh, hw = (hw + s_ - 1) >> sh;
     __syncthreads();
-    hh = max(max(halo[0], halo[2]), max(halo[4], halo[6]));
-    hw = max(max(halo[1], halo[3]), max(halo[5], halo[7]));
-    hh = __builtin_amdgcn_readfirstlane(hh);
-    hw = __builtin_amdgcn_readfirstlane(hw);
 
     // sub-tile: th x tw dx pixels (multiples of the stride), window ih x iw of dy
     const int h_lo = band * band_rows, h_hi = min(d.H, h_lo + band_rows);
@@ -507,15 +549,15 @@ __global__ __launch_bounds__(kTileThreads) __attribute__((amdgpu_waves_per_eu(4,
     const int We = max((d.W + s_ - 1) & ~(s_ - 1), 2 * s_);
     int th = s_, tw = 8;
     {
-        float best = 1e30f;
+        int best_num = 0x7fffffff / kDgradOutputs, best_den = 1;
         for (int a = RH;; a = (((a + 1) / 2) + s_ - 1) & ~(s_ - 1)) {
             for (int k = -1; k < 6; k++) {
                 const int b = k < 0 ? We : (256 >> k);  // full width, 256, 128, 64, 32, 16, 8
                 if (b > We || a * b > kDgradOutputs) continue;
                 const int ih = (a >> sh) + 2 * hh, iw = ((b >> sh) + 2 * hw) | 1;
                 if (ih * iw > dgrad_plane_elems<T>()) continue;
-                const float cost = (float)(ih * iw + 1536) / (float)(a * b);
-                if (cost < best) best = cost, th = a, tw = b;
+                const int num = ih * iw + 1536, den = a * b;
+                if (num * best_den < best_num * den) best_num = num, best_den = den, th = a, tw = b;
             }
             if (a <= s_) break;
         }
@@ -532,6 +574,7 @@ __global__ __launch_bounds__(kTileThreads) __attribute__((amdgpu_waves_per_eu(4,
         int eh, ew, fh, fw;
         const int cls = tap_class(stid, eh, ew);
         int rank = 0;
+#pragma unroll 8
         for (int t = 0; t < K; t++) {
             const int other = tap_class(t, fh, fw);
             rank += (other < cls || (other == cls && t < (int)stid)) ? 1 : 0;
@@ -540,6 +583,7 @@ __global__ __launch_bounds__(kTileThreads) __attribute__((amdgpu_waves_per_eu(4,
     }
     if ((int)stid <= ncls) {
         int below = 0, fh, fw;
+#pragma unroll 8
         for (int t = 0; t < K; t++) below += tap_class(t, fh, fw) < (int)stid ? 1 : 0;
         mystart[stid] = below;
     }
@@ -656,7 +700,7 @@ int launch_tile_dgrad_strided_src(const void *dy, const float *w, const void *ta
     const long grid = 8L * (((long)d.N * nbands + 7) / 8) * nslices;
     if (grid > 0x7fffffffL) return DWO_ERR_BAD_SHAPE;
     tile_dgrad_strided_kernel<T, Src><<<dim3((unsigned)grid), dim3(kTileThreads), lds, st>>>(
-        {(const T *)dy}, w, taps_dhdw(taps), (T *)dx, d, nbands, band_rows);
+        {(const T *)dy}, w, taps_dhdw(taps), taps_extent(taps, d.C, d.K), (T *)dx, d, nbands, band_rows);
     const hipError_t e = hipGetLastError();
     return e == hipSuccess ? 0 : (int)e;
 }
@@ -698,11 +742,11 @@ inline int tile_wgrad_groups(const ConvDims &d, int *band_rows, int *nbands) {
 template <typename T, class Src>
 __global__ __launch_bounds__(kTileThreads) __attribute__((amdgpu_waves_per_eu(4, 4))) void tile_wgrad_kernel(
     typename Src::Params spx, typename Src::Params spy, const int8_t *__restrict__ dhdw,
-    float *__restrict__ part, ConvDims d, int nbands, int band_rows, int G, int slots_log2) {
+    const int8_t *__restrict__ extent, float *__restrict__ part, ConvDims d, int nbands, int band_rows,
+    int G, int slots_log2) {
     extern __shared__ float lds_f[];
     T *planes = reinterpret_cast<T *>(lds_f);
     float *ldy = reinterpret_cast<float *>(planes + kSliceCh * tile_plane_elems<T>());  // [ch][th * tw]
-    int *halo = reinterpret_cast<int *>(ldy + kSliceCh * kTileOutputs);          // [ch][2]
 
     const int nslices = (d.C + kSliceCh - 1) / kSliceCh;
     const int g = blockIdx.x % 8 + 8 * (blockIdx.x / 8 / nslices);
@@ -716,22 +760,14 @@ __global__ __launch_bounds__(kTileThreads) __attribute__((amdgpu_waves_per_eu(4,
     const int ts = stid & (slots - 1), prt = stid >> slots_log2;
 
     const int8_t *mytaps = dhdw + (size_t)c * K * 2;
-    int hh = 0, hw = 0;
-    for (int s = 0; s < K; s++) {
-        hh = max(hh, abs((int)mytaps[2 * s]));
-        hw = max(hw, abs((int)mytaps[2 * s + 1]));
-    }
-    if (stid == 0) halo[sub * 2] = hh, halo[sub * 2 + 1] = hw;
-    __syncthreads();
-    hh = max(max(halo[0], halo[2]), max(halo[4], halo[6]));
-    hw = max(max(halo[1], halo[3]), max(halo[5], halo[7]));
-    hh = __builtin_amdgcn_readfirstlane(hh);
-    hw = __builtin_amdgcn_readfirstlane(hw);
+    int hh, hw;
+    slice_extent(extent, c0, d.C, hh, hw);
     const int rstep = hh == 0 ? s_ : 1, cstep = hw == 0 ? s_ : 1;
-    const int srow = s_ / rstep, scol = s_ / cstep;
+    const int srow = hh == 0 ? 1 : s_, scol = hw == 0 ? 1 : s_;
     // this thread's tap, in plane rows and columns (spare slots repeat tap 0 and are dropped)
-    const int my_dh = ts < K ? (int)mytaps[2 * ts] / rstep : 0;
-    const int my_dw = ts < K ? (int)mytaps[2 * ts + 1] / cstep : 0;
+    // (the steps exceed 1 only where every offset of the slice is 0: no division needed)
+    const int my_dh = ts < K ? (int)mytaps[2 * ts] : 0;
+    const int my_dw = ts < K ? (int)mytaps[2 * ts + 1] : 0;
 
     const T *plane = planes + sub * tile_plane_elems<T>();
     const float *mydy = ldy + sub * kTileOutputs;
@@ -886,7 +922,8 @@ int launch_tile_wgrad_src(const void *x, const void *dy, const void *taps, float
     int slots_log2 = 0;
     while ((1 << slots_log2) < d.K) slots_log2++;
     tile_wgrad_kernel<T, Src><<<dim3((unsigned)(G * nslices)), dim3(kTileThreads), lds, st>>>(
-        {(const T *)x}, {(const T *)dy}, taps_dhdw(taps), part, d, nbands, band_rows, G, slots_log2);
+        {(const T *)x}, {(const T *)dy}, taps_dhdw(taps), taps_extent(taps, d.C, d.K), part, d, nbands,
+        band_rows, G, slots_log2);
     const hipError_t e = hipGetLastError();
     return e == hipSuccess ? 0 : (int)e;
 }
