@@ -371,14 +371,6 @@ int dwo_build_taps(const float *theta_host, int C, int K, void *taps_host) {
                        dhdw[((size_t)c * K + s) * 2 + 1] == canon_dw(o, K, s);
             if (same) cls[c] = o;
         }
-        // ... or one of them in reverse order (the layers turned by 90 degrees reach 180 .. 247.5)
-        for (int o = 0; o < 8 && cls[c] < 0; o++) {
-            bool same = true;
-            for (int s = 0; s < K && same; s++)
-                same = dhdw[((size_t)c * K + s) * 2] == canon_dh(o, K, K - 1 - s) &&
-                       dhdw[((size_t)c * K + s) * 2 + 1] == canon_dw(o, K, K - 1 - s);
-            if (same) cls[c] = o + 8;
-        }
     }
     // channel order that cycles through the classes: 0, 1, .., 7, non-canonical, 0, 1, ..
     hdr[6] = hdr[5] + (int32_t)taps_class_bytes(C);
@@ -389,7 +381,7 @@ int dwo_build_taps(const float *theta_host, int C, int K, void *taps_host) {
         for (int k = 0; k < 9 && placed < C; k++) {
             const int want = k < 8 ? k : -1;
             int c = next[k];
-            while (c < C && class_orientation(cls[c]) != want) c++;
+            while (c < C && cls[c] != want) c++;
             next[k] = c + 1;
             if (c < C) order[placed++] = c;
         }

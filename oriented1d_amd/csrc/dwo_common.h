@@ -36,11 +36,6 @@ __host__ __device__ inline const int8_t *taps_dhdw(const void *blob) {
 __host__ __device__ inline size_t taps_class_bytes(int C) {
     return ((size_t)C * 4 + 15) & ~(size_t)15;
 }
-// Class word of a channel: -1 when its taps match no compile-time pattern, else the canonical
-// orientation o (0..7, k * 22.5 degrees) plus 8 when the taps are that pattern in reverse order
-// (the angle plus 180 degrees): the same line of positions, with the weights running the other way.
-__host__ __device__ inline int class_orientation(int cls) { return cls < 0 ? -1 : (cls & 7); }
-__host__ __device__ inline bool class_reversed(int cls) { return cls >= 8; }
 __host__ __device__ inline const int32_t *taps_class(const void *blob, int C, int K) {
     return reinterpret_cast<const int32_t *>(reinterpret_cast<const int8_t *>(blob) +
                                              kTapsHeaderBytes + taps_dhdw_bytes(C, K));

@@ -129,14 +129,14 @@ struct NhwcCtx {
 template <int O, int OP, typename T, int K, int H, int W>
 __device__ __forceinline__ void nhwc_canonical(NhwcCtx<T, K, H, W> &ctx, const float *__restrict__ wt,
                                                const float *__restrict__ bias, int c, int sub,
-                                               unsigned stid, int n0, bool rev) {
+                                               unsigned stid, int n0) {
     using Ctx = NhwcCtx<T, K, H, W>;
     constexpr int L = tile_L<H, W>(O);
     constexpr int PBI = Ctx::PBI, NTS = Ctx::NT / kSliceCh, PLS = Ctx::PLS;
     using G = Geo<O, K, L, H, W>;
     constexpr int ITERS = (PBI * G::IPP + NTS - 1) / NTS;
     ChannelTaps<G, OP, T, K, false> taps;
-    taps.load(wt, bias, c, rev);
+    taps.load(wt, bias, c);
     float *planes = ctx.lds + sub * PBI * PLS;
 
     ctx.zero_fill();
@@ -273,18 +273,17 @@ __global__ __launch_bounds__((NhwcTile<H, W>::NT)) void nhwc_plane_kernel(
     const int32_t *cls = taps_class(blob, C, K) + c0;
 #pragma unroll
     for (int ch = 0; ch < kSliceCh; ch++) {
-        ctx.g[ch] = geo_rt<K, H, W>(class_orientation(cls[ch]));
+        ctx.g[ch] = geo_rt<K, H, W>(cls[ch]);
     }
     const int sub = __builtin_amdgcn_readfirstlane(threadIdx.x / NTS);
     const unsigned stid = threadIdx.x % NTS;
     const int c = c0 + sub;
     const int mine = cls[sub];
-#define DWO_CASE(O)                                                                  \
-    case O:                                                                          \
-        nhwc_canonical<O, OP, T, K, H, W>(ctx, wt, bias, c, sub, stid, n0,            \
-                                          class_reversed(mine));                     \
+#define DWO_CASE(O)                                                             \
+    case O:                                                                     \
+        nhwc_canonical<O, OP, T, K, H, W>(ctx, wt, bias, c, sub, stid, n0);      \
         break;
-    switch (class_orientation(mine)) {
+    switch (mine) {
         DWO_CASE(0)
         DWO_CASE(1)
         DWO_CASE(2)
@@ -601,19 +600,18 @@ __global__ __launch_bounds__((NhwcTile<H, W>::NT)) void nhwc_plane_wgrad_kernel(
     const int32_t *cls = taps_class(blob, C, K) + c0;
 #pragma unroll
     for (int ch = 0; ch < kSliceCh; ch++) {
-        ctx.g[ch] = geo_rt<K, H, W>(class_orientation(cls[ch]));
-        ctx.split[ch] = (short)split_row<K, H, W>(class_orientation(cls[ch]));
+        ctx.g[ch] = geo_rt<K, H, W>(cls[ch]);
+        ctx.split[ch] = (short)split_row<K, H, W>(cls[ch]);
     }
     const int sub = __builtin_amdgcn_readfirstlane(threadIdx.x / NTS);
     const unsigned stid = threadIdx.x % NTS;
     const int c = c0 + sub;
     const int mine = cls[sub];
-    out.rev = class_reversed(mine);
 #define DWO_CASE(O)                                                                     \
     case O:                                                                             \
         nhwc_canonical_wgrad<O, T, K, H, W>(ctx, out, c, sub, stid, n0, group);          \
         break;
-    switch (class_orientation(mine)) {
+    switch (mine) {
         DWO_CASE(0)
         DWO_CASE(1)
         DWO_CASE(2)
@@ -642,7 +640,7 @@ int launch_nhwc_plane_wgrad(const void *x, const void *dy, const void *taps, flo
     const int groups = plane_groups(N, nslices, PBI, slots);
     *groups_out = groups;
     nhwc_plane_wgrad_kernel<T, K, H, W><<<dim3(nslices * groups), dim3(NT), lds, st>>>(
-        (const T *)x, (const T *)dy, taps, WgradOut{part, dw, db, groups, 0}, N, C);
+        (const T *)x, (const T *)dy, taps, WgradOut{part, dw, db, groups}, N, C);
     const hipError_t e = hipGetLastError();
     return e == hipSuccess ? 0 : (int)e;
 }

@@ -373,13 +373,11 @@ struct ChannelTaps {
     unsigned wp[NPAIR];
     float bv;
 
-    // rev: the channel's taps are G's pattern in reverse order, so its weights are read backwards
     __device__ __forceinline__ void load(const float *__restrict__ wt, const float *__restrict__ bias,
-                                         int c, bool rev) {
+                                         int c) {
         const float *wc = wt + (size_t)c * K;
-        const bool back = (OP == OP_DGRAD) != rev;
 #pragma unroll
-        for (int s = 0; s < K; s++) wv[s] = wc[back ? K - 1 - s : s];
+        for (int s = 0; s < K; s++) wv[s] = wc[OP == OP_DGRAD ? K - 1 - s : s];
         static_for<K>([&](auto s) {
             constexpr int r = G::plan.rep[s];
             if constexpr (r >= 0 && r != s) wv[r] += wv[s];
@@ -443,7 +441,7 @@ template <int O, int OP, typename T, int K, int H, int W>
 __device__ __forceinline__ void run_canonical(const T *__restrict__ src, const float *__restrict__ wt,
                                               const float *__restrict__ bias, T *__restrict__ dst,
                                               float *lds, int c, int C, int n0, int n1,
-                                              ConvStagers<T, H, W> &sg, bool rev) {
+                                              ConvStagers<T, H, W> &sg) {
     constexpr int L = tile_L<H, W>(O);
     constexpr int PB = Tile<H, W>::PB, NT = Tile<H, W>::NT;
     constexpr bool PAIR = use_pairs<T, O, W>();
@@ -454,7 +452,7 @@ __device__ __forceinline__ void run_canonical(const T *__restrict__ src, const f
     const unsigned pstride = (unsigned)C * (H * W);  // elements between images of one channel
 
     ChannelTaps<G, OP, T, K, PAIR> taps;
-    taps.load(wt, bias, c, rev);
+    taps.load(wt, bias, c);
 
     // zero the staging area once; interiors are overwritten per batch, halos stay zero
     for (unsigned i = tid; i < PB * PLS; i += NT) lds[i] = 0.f;
@@ -640,9 +638,7 @@ __device__ __forceinline__ float wave_sum_dpp(float v) {
 struct WgradOut {
     float *part, *dw, *db;
     int NG;
-    int rev;  // set per channel by the kernel: sums arrive in reverse tap order
     __device__ __forceinline__ void put(int c, int s, int group, int K, float t) const {
-        if (rev && s < K) s = K - 1 - s;
         if (NG > 1)
             part[((size_t)c * (K + 1) + s) * NG + group] = t;
         else if (s < K)
@@ -819,12 +815,11 @@ __global__ __launch_bounds__((Tile<H, W>::NT)) __attribute__((amdgpu_waves_per_e
     int n0, n1;
     group_range<Tile<H, W>::PB>(N, NG, group, n0, n1);
     const int cls = taps_class(blob, C, K)[c];
-    out.rev = class_reversed(cls);
 #define DWO_CASE(O)                                                                      \
     case O:                                                                              \
         run_canonical_wgrad<O, T, K, H, W>(x, dy, out, lds, c, C, n0, n1, group);         \
         break;
-    switch (class_orientation(cls)) {
+    switch (cls) {
         DWO_CASE(0)
         DWO_CASE(1)
         DWO_CASE(2)
@@ -864,10 +859,9 @@ __global__ __launch_bounds__((Tile<H, W>::NT)) __attribute__((amdgpu_waves_per_e
     const int cls = taps_class(blob, C, K)[c];
 #define DWO_CASE(O)                                                                  \
     case O:                                                                          \
-        run_canonical<O, OP, T, K, H, W>(src, wt, bias, dst, lds, c, C, n0, n1, sg,   \
-                                         class_reversed(cls));                        \
+        run_canonical<O, OP, T, K, H, W>(src, wt, bias, dst, lds, c, C, n0, n1, sg);  \
         break;
-    switch (class_orientation(cls)) {
+    switch (cls) {
         DWO_CASE(0)
         DWO_CASE(1)
         DWO_CASE(2)
@@ -926,7 +920,7 @@ int launch_plane_wgrad(const void *x, const void *dy, const void *taps, float *p
     const int groups = plane_groups(N, C, Tile<H, W>::PB, slots);
     *groups_out = groups;
     plane_wgrad_kernel<T, K, H, W><<<dim3(C * groups), dim3(NT), lds, st>>>(
-        (const T *)x, (const T *)dy, taps, WgradOut{part, dw, db, groups, 0}, N, C);
+        (const T *)x, (const T *)dy, taps, WgradOut{part, dw, db, groups}, N, C);
     const hipError_t e = hipGetLastError();
     return e == hipSuccess ? 0 : (int)e;
 }

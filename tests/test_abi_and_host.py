@@ -91,21 +91,6 @@ def test_tap_table_channel_order_cycles_through_classes(layout):
         assert all(sorted(r.tolist()) == [-1] + list(range(8)) for r in first)
 
 
-def test_tap_table_marks_reversed_canonical_patterns():
-    """An angle of k * 22.5 + 180 degrees walks a canonical line backwards: class word o + 8."""
-    from parity_util import canonical_theta
-    C, K = 16, 31
-    theta = canonical_theta(C)
-    theta[8:] += np.float32(math.pi)
-    blob = op.build_taps(torch.from_numpy(theta.astype(np.float32)), C, K).numpy()
-    hdr = blob[:32].view(np.int32)
-    cls = blob[hdr[5]:hdr[5] + 4 * C].view(np.int32)
-    assert cls[:8].tolist() == list(range(8))
-    assert cls[8:].tolist() == [o + 8 for o in range(8)]
-    dh, dw = op.taps_to_numpy(torch.from_numpy(blob), C, K)
-    assert (dh[8:] == dh[:8, ::-1]).all() and (dw[8:] == dw[:8, ::-1]).all()
-
-
 def test_module_contract():
     C, K = 16, 31
     angles = [math.pi * (c % 8) / 8 for c in range(C)]
