@@ -168,6 +168,32 @@ def test_random_angles_ragged_shapes(oracle, nhwc):
         _case(oracle, N, C, H, W, K, 1, torch.float32, nhwc, theta, seed=N * C + H)
 
 
+@pytest.mark.parametrize("nhwc", [False, True], ids=["nchw", "nhwc"])
+@pytest.mark.parametrize("stride", [2, 4])
+def test_strided_ragged_shapes_random_angles(oracle, stride, nhwc):
+    """Strided fprop, dgrad by residue classes and wgrad at degenerate extents (single rows and
+    columns, extents below the stride), odd channel counts, random angles."""
+    rng = np.random.default_rng(100 + stride)
+    for (N, C, H, W, K) in [(1, 1, 1, 1, 31), (2, 3, 1, 9, 7), (2, 6, 9, 1, 15), (1, 9, 3, 2, 31),
+                            (2, 12, 33, 17, 31), (1, 4, 70, 61, 27), (3, 8, 5, 130, 13)]:
+        if nhwc and C % 4 != 0 and K not in (7, 13, 15, 27, 31):
+            continue
+        theta = rng.uniform(-math.pi, 2 * math.pi, C).astype(np.float32)
+        _case(oracle, N, C, H, W, K, stride, torch.float32, nhwc, theta, seed=N * C + H + stride)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("nhwc", [False, True], ids=["nchw", "nhwc"])
+def test_largest_kernel_size(oracle, nhwc, dtype):
+    """K = 63, the largest the tap table holds: 16-bit activations run on the tile kernels, fp32
+    (whose smallest window would not fit an LDS plane) on the generic ones."""
+    rng = np.random.default_rng(63)
+    theta = rng.uniform(0, math.pi, 8).astype(np.float32)
+    theta[:3] = [0.0, math.pi / 2, math.pi / 4]
+    _case(oracle, 2, 8, 40, 37, 63, 1, dtype, nhwc, theta, seed=63)
+    _case(oracle, 1, 8, 40, 37, 63, 2, dtype, nhwc, theta, seed=64)
+
+
 def test_wgrad_is_deterministic():
     C, K = 96, 31
     g = torch.Generator(device="cuda").manual_seed(5)
