@@ -266,6 +266,53 @@ def main():
                 "ops": {k: [v["us"], v["frac_hbm"]] for k, v in r["detail"].items()}}
             torch.cuda.empty_cache()
 
+    # ------------------------------------------------------------------ shapes without planes
+    # Per-kernel times of the tile kernels (any extent, stride and layout): the two stem
+    # convolutions of the networks at batch 128 (NHWC, stride 2) and the stage shapes of a 512 x 512
+    # input at batch 8 (NCHW), bf16, the networks' contiguous-group angles.
+    other_shapes = {}
+    if not args.no_extra_sweeps and not args.only:
+        for tag, (N_, C_, HW_, st_, lay_) in (
+                ("stem1 128x64x224 s2 nhwc", (128, 64, 224, 2, "nhwc")),
+                ("stem2 128x64x112 s2 nhwc", (128, 64, 112, 2, "nhwc")),
+                ("8x96x128 nchw", (8, 96, 128, 1, "nchw")), ("8x192x64 nchw", (8, 192, 64, 1, "nchw")),
+                ("8x384x32 nchw", (8, 384, 32, 1, "nchw")), ("8x768x16 nchw", (8, 768, 16, 1, "nchw"))):
+            nhwc = lay_ == "nhwc"
+            PQ = -(-HW_ // st_)
+            g = torch.Generator(device=dev).manual_seed(1)
+            xs = (N_, HW_, HW_, C_) if nhwc else (N_, C_, HW_, HW_)
+            ys = (N_, PQ, PQ, C_) if nhwc else (N_, C_, PQ, PQ)
+            x = torch.randn(xs, device=dev, generator=g).to(torch.bfloat16)
+            dy = torch.randn(ys, device=dev, generator=g).to(torch.bfloat16)
+            w2 = (torch.randn(C_, KSIZE, device=dev, generator=g) * 0.02).contiguous()
+            taps = op.build_taps(torch.from_numpy(theta_for(C_, "grouped")), C_, KSIZE).to(dev)
+            y, dx = torch.empty_like(dy), torch.empty_like(x)
+            dw = torch.empty(C_, KSIZE, device=dev)
+            nb = lib.dwo_wgrad_scratch_bytes(N_, C_, HW_, HW_, KSIZE, st_, 1, int(nhwc))
+            scr = torch.empty(max(nb, 16), dtype=torch.uint8, device=dev)
+            dims = (N_, C_, HW_, HW_, KSIZE, st_, 1, int(nhwc), stream_h)
+            fns = {"fprop": (lambda a=(vp(x), vp(w2), None, vp(taps), vp(y)) + dims: lib.dwo_fprop(*a)),
+                   "dgrad": (lambda a=(vp(dy), vp(w2), vp(taps), vp(dx)) + dims: lib.dwo_dgrad(*a)),
+                   "wgrad": (lambda a=(vp(dy), vp(x), vp(taps), vp(dw), None, vp(scr), nb) + dims:
+                             lib.dwo_wgrad(*a))}
+            row = {}
+            torch.cuda.synchronize()  # inputs were made on torch's stream, the calls run on `stream`
+            for name, fn in fns.items():
+                _lib.check(fn(), "dwo_" + name)
+                torch.cuda.synchronize()
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record(stream)
+                for _ in range(10):
+                    fn()
+                e1.record(stream)
+                torch.cuda.synchronize()
+                us = e0.elapsed_time(e1) * 100.0
+                ab = algorithmic_bytes(name, N_, C_, HW_, HW_, KSIZE, 2, st_)
+                row[name] = [round(us, 1), round(ab / us / 1e3 / HBM_PEAK_GBS, 4)]
+            other_shapes[tag] = row
+            del x, dy, y, dx, scr
+            torch.cuda.empty_cache()
+
     # ------------------------------------------------------------------ CPU baseline (oracle)
     cpu, cpu_all = None, None
     if not args.no_cpu_baseline:
@@ -455,7 +502,7 @@ def main():
                    "algorithmic_bytes_per_step": step_bytes},
         "frac_hbm_peak": round(value / HBM_PEAK_GBS, 4),
         "detail": detail, "roofline": roofline, "cpu_baseline": cpu,
-        "cpu_baseline_all_threads": cpu_all, "other_configs": others,
+        "cpu_baseline_all_threads": cpu_all, "other_configs": others, "other_shapes_bf16": other_shapes,
         "convnext_t_1d": model_info, "training_configs": train_info,
     }
     print(json.dumps(out))
