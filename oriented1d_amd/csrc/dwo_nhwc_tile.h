@@ -1,18 +1,22 @@
-// fprop (and, with reversed weights, stride-1 dgrad) for any plane extent, stride and kernel
-// size: the stem convolutions of the ConvNeXt-1D networks (NHWC, 224 -> 112 -> 56, stride 2),
-// the stages of inputs other than 224 x 224 (NCHW), and every other shape without compile-time
-// planes.  NHWC needs a channel count that is a multiple of 4.  Described for NHWC; NCHW differs
-// only in how the window is loaded and the results are stored (PlaneSource).
+// Tile kernels: fprop, dgrad and wgrad for any plane extent, stride, kernel size and angle, in
+// both layouts: the stem convolutions of the ConvNeXt-1D networks (NHWC, 224 -> 112 -> 56,
+// stride 2), the stages of inputs other than 224 x 224 (NCHW), and every other shape without
+// compile-time planes.  NHWC needs a channel count that is a multiple of 4.  The layouts differ
+// only in how a window is loaded (SliceSource, PlaneSource; PointwiseSource applies the stem's
+// pointwise projection on the way in) and in how results are stored (tile_flush).
 //
-// A workgroup owns four consecutive channels of a band of output rows of one image and walks
-// the band in sub-tiles.  Per sub-tile it loads the pixel slices of the input window (8 or 16
-// bytes per pixel), stores them as one plane per channel in LDS in the activation's own type
-// (out-of-image positions as zeros), lets sub-group k (128 threads) evaluate channel k's taps
-// for the sub-tile's outputs from that plane, and writes the results back as pixel slices.
-// The sub-tile shape is chosen per workgroup from its channels' tap extents: wide row strips
-// for near-horizontal taps, tall column strips for near-vertical ones, squares in between, so
-// the window read per output stays small for every orientation.  The extents are bounded by
-// K / 2 in each direction, whatever the angles.
+// fprop (nhwc_tile_fprop_kernel; with reversed weights also dgrad at stride 1): a workgroup owns
+// four consecutive channels of a band of output rows of one image and walks the band in
+// sub-tiles.  Per sub-tile it loads the input window, stores it as one plane per channel in LDS in
+// the activation's own type (out-of-image positions as zeros), lets sub-group k (128 threads)
+// evaluate channel k's taps for the sub-tile's outputs from that plane, and writes the results
+// out.  The sub-tile shape is chosen per workgroup from its channels' tap extents: wide row
+// strips for near-horizontal taps, tall column strips for near-vertical ones, squares in
+// between, so the window read per output stays small for every orientation.  The extents are
+// bounded by K / 2 in each direction, whatever the angles.
+//
+// tile_dgrad_strided_kernel (strides 2 and 4) and tile_wgrad_kernel are described where they
+// are defined.
 #pragma once
 
 #include <type_traits>
