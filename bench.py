@@ -237,7 +237,7 @@ def main():
     # scaled by what the same counter reads for a plain copy of known size (summary and the
     # commands under profiles/dwoconv1d_stage_sweep_f32_nchw_hbm_traffic.md); only valid for
     # the configuration it was measured on.
-    measured_traffic = {("f32", "nchw", "roundrobin"): 160382566}
+    measured_traffic = {("f32", "nchw", "roundrobin"): 160340699}
 
     dom = detail.get("96x56:fprop")
     roofline = None
