@@ -130,14 +130,14 @@ def main():
                 nb = lib.dwo_wgrad_scratch_bytes(BATCH, C, HW, HW, KSIZE, 1, dt_code, lay_code)
                 scr = torch.empty(max(nb, 16), dtype=torch.uint8, device=dev)
                 keep.extend([x, dy, w2, taps, y, dx, dw, scr])
-                dims = (BATCH, C, HW, HW, KSIZE, 1, dt_code, lay_code, stream_h)
+                dims = (BATCH, C, HW, HW, KSIZE, 1, dt_code, lay_code)
                 fa = (vp(x), vp(w2), None, vp(taps), vp(y)) + dims
                 da = (vp(dy), vp(w2), vp(taps), vp(dx)) + dims
                 wa = (vp(dy), vp(x), vp(taps), vp(dw), None, vp(scr), nb) + dims
                 per_stage.append({
-                    "fprop": (lambda a=fa: lib.dwo_fprop(*a)),
-                    "dgrad": (lambda a=da: lib.dwo_dgrad(*a)),
-                    "wgrad": (lambda a=wa: lib.dwo_wgrad(*a)),
+                    "fprop": (lambda sh=stream_h, a=fa: lib.dwo_fprop(*a, sh)),
+                    "dgrad": (lambda sh=stream_h, a=da: lib.dwo_dgrad(*a, sh)),
+                    "wgrad": (lambda sh=stream_h, a=wa: lib.dwo_wgrad(*a, sh)),
                 })
             calls.append(per_stage)
         for ops in calls[0]:  # one checked pass: any launch error surfaces here
@@ -153,7 +153,7 @@ def main():
 
         step_bytes = sum(algorithmic_bytes(o, BATCH, C, HW, HW, KSIZE, b)
                          for C, HW in STAGES for o in ("fprop", "dgrad", "wgrad"))
-        ms_per_step, ms_eager = None, None
+        ms_per_step, ms_eager, ms_branches, ms_graph = None, None, None, None
         if steps > 0:
             for i in range(warmup):
                 step(i)
@@ -180,7 +180,37 @@ def main():
                 for i in range(steps):
                     graphs[i % nsets].replay()
                 torch.cuda.synchronize()
-                ms_per_step = (time.perf_counter() - t0) * 1e3 / steps
+                ms_graph = (time.perf_counter() - t0) * 1e3 / steps
+                # the step time reported is the faster of the two complete measurements
+                ms_per_step = min(ms_eager, ms_graph)
+                del graphs
+                # For information (not `value`): the same step with fprop, dgrad and wgrad of a
+                # shape on three parallel branches of the graph (they do not depend on each other;
+                # in a training step dgrad and wgrad of a layer do not either), so the fill and
+                # drain of one kernel overlaps its neighbours'.
+                side = [torch.cuda.Stream(dev), torch.cuda.Stream(dev)]
+                side_h = [ctypes.c_void_p(s_.cuda_stream) for s_ in side]
+                graphs = []
+                for i in range(nsets):
+                    gr = torch.cuda.CUDAGraph()
+                    with torch.cuda.graph(gr, stream=stream):
+                        for s_ in side:
+                            s_.wait_stream(stream)
+                        for ops in calls[i % nsets]:
+                            ops["fprop"]()
+                            ops["dgrad"](side_h[0])
+                            ops["wgrad"](side_h[1])
+                        for s_ in side:
+                            stream.wait_stream(s_)
+                    graphs.append(gr)
+                for i in range(warmup):
+                    graphs[i % nsets].replay()
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                for i in range(steps):
+                    graphs[i % nsets].replay()
+                torch.cuda.synchronize()
+                ms_branches = (time.perf_counter() - t0) * 1e3 / steps
                 del graphs
 
         # per-kernel timings: HIP events on the launch stream (torch's current stream is the
@@ -214,7 +244,8 @@ def main():
                 if warm:
                     detail[key]["warm_us"] = round(timed(name, si, True), 2)
         copy_src = keep[0]
-        res = {"ms_per_step": ms_per_step, "ms_per_step_eager": ms_eager, "detail": detail,
+        res = {"ms_per_step": ms_per_step, "ms_per_step_eager": ms_eager,
+               "ms_per_step_branches": ms_branches, "ms_per_step_graph": ms_graph, "detail": detail,
                "nsets": nsets,
                "step_bytes": step_bytes, "copy_src": copy_src if args.calibration_copy else None}
         return res
@@ -496,9 +527,14 @@ def main():
                                "(C=96@56x56, 192@28x28, 384@14x14, 768@7x7), batch 64, K=31, "
                                "8 orientations %s, stride 1" % args.theta,
                    "layout": args.layout, "buffer_sets": nsets,
-                   "launch": ("hipGraph replay of the step's 12 C-ABI calls (one graph per "
-                              "buffer set)" if args.graph else "eager C-ABI calls"),
+                   "launch": "the faster of eager C-ABI calls and hipGraph replay of the step's 12 "
+                             "calls (one graph per buffer set); both are listed",
+                   "ms_per_step_graph": (round(main_res["ms_per_step_graph"], 4)
+                                         if main_res["ms_per_step_graph"] else None),
                    "ms_per_step_eager": round(main_res_eager, 4),
+                   "ms_per_step_parallel_branches": (
+                       round(main_res["ms_per_step_branches"], 4)
+                       if main_res["ms_per_step_branches"] else None),
                    "algorithmic_bytes_per_step": step_bytes},
         "frac_hbm_peak": round(value / HBM_PEAK_GBS, 4),
         "detail": detail, "roofline": roofline, "cpu_baseline": cpu,
