@@ -254,6 +254,7 @@ def main():
                      args.kernel_iters, args.kernel_repeats, args.only, warm=True)
     ms_per_step, detail = main_res["ms_per_step"], main_res["detail"]
     main_res_eager = main_res["ms_per_step_eager"]
+    main_res_graph, main_res_branches = main_res["ms_per_step_graph"], main_res["ms_per_step_branches"]
     nsets, step_bytes = main_res["nsets"], main_res["step_bytes"]
     value = step_bytes / (ms_per_step * 1e-3) / 1e9
 
@@ -529,12 +530,10 @@ def main():
                    "layout": args.layout, "buffer_sets": nsets,
                    "launch": "the faster of eager C-ABI calls and hipGraph replay of the step's 12 "
                              "calls (one graph per buffer set); both are listed",
-                   "ms_per_step_graph": (round(main_res["ms_per_step_graph"], 4)
-                                         if main_res["ms_per_step_graph"] else None),
+                   "ms_per_step_graph": round(main_res_graph, 4) if main_res_graph else None,
                    "ms_per_step_eager": round(main_res_eager, 4),
-                   "ms_per_step_parallel_branches": (
-                       round(main_res["ms_per_step_branches"], 4)
-                       if main_res["ms_per_step_branches"] else None),
+                   "ms_per_step_parallel_branches": (round(main_res_branches, 4)
+                                                     if main_res_branches else None),
                    "algorithmic_bytes_per_step": step_bytes},
         "frac_hbm_peak": round(value / HBM_PEAK_GBS, 4),
         "detail": detail, "roofline": roofline, "cpu_baseline": cpu,
