@@ -194,6 +194,32 @@ def test_largest_kernel_size(oracle, nhwc, dtype):
     _case(oracle, 1, 8, 40, 37, 63, 2, dtype, nhwc, theta, seed=64)
 
 
+@pytest.mark.parametrize("seed", [11, 12, 13])
+def test_randomized_shapes_all_paths(oracle, seed):
+    """Seeded random draws over batch, channels, extents, kernel size, stride, element type,
+    layout and angle assignment (arbitrary, round-robin canonical, grouped canonical): every
+    routing decision of the C ABI gets exercised at shapes nobody picked by hand."""
+    rng = np.random.default_rng(seed)
+    for it in range(40):
+        nhwc = bool(rng.integers(2))
+        K = int(rng.choice([3, 7, 13, 15, 27, 31, 45, 63]))
+        stride = int(rng.choice([1, 1, 2, 4]))
+        N = int(rng.integers(1, 4))
+        C = int(rng.choice([1, 2, 3, 4, 5, 8, 12, 17, 32, 36]))
+        H, W = int(rng.integers(1, 90)), int(rng.integers(1, 150))
+        if rng.integers(4) == 0:
+            H, W = W, H
+        dtype = DTYPES[int(rng.integers(3))]
+        kind = int(rng.integers(3))
+        if kind == 0:
+            theta = rng.uniform(-math.pi, 2 * math.pi, C).astype(np.float32)
+        elif kind == 1:
+            theta = canonical_theta(C)
+        else:
+            theta = grouped_theta(C)
+        _case(oracle, N, C, H, W, K, stride, dtype, nhwc, theta, seed=seed * 1000 + it)
+
+
 def test_wgrad_is_deterministic():
     C, K = 96, 31
     g = torch.Generator(device="cuda").manual_seed(5)
