@@ -7,10 +7,12 @@ degrees), i.e. 12 launches of the C-ABI entry points.  Inputs are resident in HB
 timed region; buffer sets rotate so consecutive steps do not re-hit the 256 MB Infinity Cache.
 
 Prints ONE JSON line: `value` is the algorithmic GB/s of the whole step (sum of the 12
-operators' algorithmic bytes / step time); `detail` carries GB/s and the HBM-roofline
-fraction of every (shape, op); `roofline` is the dominant kernel (fprop at C=96, 56x56,
-the largest byte count), timed with events on the launch stream; `cpu_baseline` is the
-oracle's single-thread reference-order loops on a bounded sample of the same workload.
+operators' algorithmic bytes / step time, eager C-ABI calls); `detail` carries GB/s and the
+HBM-roofline fraction of every (shape, op); `roofline` is the dominant kernel, i.e. the one of
+the twelve with the longest launch, timed with events on the launch stream, and `roofline_min`
+the lowest fraction among the twelve; `cpu_baseline` is the oracle's single-thread
+reference-order loops on a bounded sample of the same workload; `table5` repeats the
+reference's own micro-benchmark (analysis/benchmark.py:19-67,84-104).
 """
 import argparse
 import json
@@ -52,8 +54,11 @@ def main():
     ap.add_argument("--kernel-repeats", type=int, default=7,
                     help="repeats of the per-kernel measurement (the median is reported)")
     ap.add_argument("--no-graph", dest="graph", action="store_false",
-                    help="time eager launches of the 12 C-ABI calls instead of replays of their "
-                         "captured graph")
+                    help="skip the two informational hipGraph timings of the step (`value` is "
+                         "always the eager C-ABI calls)")
+    ap.add_argument("--table5-iters", type=int, default=20,
+                    help="timed iterations per angle of the reference's Table-5 protocol "
+                         "(the reference uses 100); 0 skips it")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra-sweeps", action="store_true",
                     help="skip the bf16 / NHWC / grouped-angle rows (other_configs)")
@@ -85,7 +90,7 @@ def main():
     import ctypes
 
     from oriented1d_amd import _lib
-    lib = _lib.load()
+    lib = _lib.ready(dev)  # dwo_init: every kernel set up before anything is captured or timed
     # everything runs on one side stream: its handle is what the C ABI launches on, what the
     # timing events are recorded on, and what the step graphs are captured from
     stream = torch.cuda.Stream(dev)
@@ -140,10 +145,15 @@ def main():
                     "wgrad": (lambda sh=stream_h, a=wa: lib.dwo_wgrad(*a, sh)),
                 })
             calls.append(per_stage)
-        for ops in calls[0]:  # one checked pass: any launch error surfaces here
-            for name, fn in ops.items():
-                _lib.check(fn(), "dwo_" + name)
-        torch.cuda.synchronize()
+        def checked_pass():
+            """Every call of every buffer set once, with its status checked."""
+            for per_stage in calls:
+                for ops in per_stage:
+                    for name, fn in ops.items():
+                        _lib.check(fn(), "dwo_" + name)
+            torch.cuda.synchronize()
+
+        checked_pass()  # any launch error surfaces here, before anything is timed
 
         def step(i):
             for ops in calls[i % nsets]:
@@ -165,8 +175,8 @@ def main():
             ms_eager = (time.perf_counter() - t0) * 1e3 / steps
             ms_per_step = ms_eager
             if args.graph:
-                # the same 12 C-ABI calls per step, captured once per buffer set and replayed:
-                # one launch per step instead of 16 kernel launches from the host
+                # For information (not `value`): the same 12 C-ABI calls per step, captured once
+                # per buffer set and replayed
                 graphs = []
                 for i in range(nsets):
                     gr = torch.cuda.CUDAGraph()
@@ -181,8 +191,6 @@ def main():
                     graphs[i % nsets].replay()
                 torch.cuda.synchronize()
                 ms_graph = (time.perf_counter() - t0) * 1e3 / steps
-                # the step time reported is the faster of the two complete measurements
-                ms_per_step = min(ms_eager, ms_graph)
                 del graphs
                 # For information (not `value`): the same step with fprop, dgrad and wgrad of a
                 # shape on three parallel branches of the graph (they do not depend on each other;
@@ -212,6 +220,7 @@ def main():
                 torch.cuda.synchronize()
                 ms_branches = (time.perf_counter() - t0) * 1e3 / steps
                 del graphs
+            checked_pass()  # the timed calls discard their status: re-check every set afterwards
 
         # per-kernel timings: HIP events on the launch stream (torch's current stream is the
         # one passed to the C ABI), median over the repeats
@@ -265,20 +274,36 @@ def main():
             dstc.copy_(src)
         torch.cuda.synchronize()
 
-    # HBM bytes per launch of the dominant kernel from rocprofv3 FETCH_SIZE + WRITE_SIZE, each
-    # scaled by what the same counter reads for a plain copy of known size (summary and the
-    # commands under profiles/dwoconv1d_stage_sweep_f32_nchw_hbm_traffic.md); only valid for
-    # the configuration it was measured on.
-    measured_traffic = {("f32", "nchw", "roundrobin"): 160340699}
+    # HBM bytes per launch from rocprofv3 FETCH_SIZE + WRITE_SIZE, each scaled by what the same
+    # counter reads for a plain copy of known size: the figures and the commands that produced
+    # them are committed under profiles/ (a .md summary and the same numbers as .json); only
+    # valid for the configuration they were measured on.
+    traffic = {}
+    tpath = os.path.join(ROOT, "profiles", "dwoconv1d_stage_sweep_%s_%s_hbm_traffic.json"
+                         % (args.dtype, args.layout))
+    if args.theta == "roundrobin" and os.path.exists(tpath):
+        with open(tpath) as fh:
+            traffic = json.load(fh).get("traffic_bytes_per_launch", {})
 
-    dom = detail.get("96x56:fprop")
-    roofline = None
-    if dom:
-        roofline = {"bound": "hbm", "kernel": "fprop C=96 56x56 N=64 %s %s" % (args.dtype, args.layout),
+    # the dominant kernel is the one of the twelve with the longest launch
+    roofline, roofline_min = None, None
+    if detail:
+        dom_key = max(detail, key=lambda k: detail[k]["us"])
+        dom = detail[dom_key]
+        C_, rest = dom_key.split("x")
+        HW_, op_ = rest.split(":")
+        roofline = {"bound": "hbm",
+                    "kernel": "%s C=%s %sx%s N=%d %s %s" % (op_, C_, HW_, HW_, BATCH, args.dtype,
+                                                           args.layout),
                     "achieved": dom["GB/s"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
                     "frac": round(dom["GB/s"] / HBM_PEAK_GBS, 4),
-                    "traffic": measured_traffic.get((args.dtype, args.layout, args.theta)),
+                    "traffic": traffic.get(dom_key),
                     "launch_us": dom["us"], "algorithmic_bytes": dom["bytes"]}
+        low_key = min(detail, key=lambda k: detail[k]["frac_hbm"])
+        roofline_min = {"kernel": low_key, "frac": detail[low_key]["frac_hbm"],
+                        "launch_us": detail[low_key]["us"],
+                        "ops_at_or_above_0.60": sum(v["frac_hbm"] >= 0.6 for v in detail.values()),
+                        "ops": len(detail)}
 
     # ------------------------------------------------------------------ the other rows
     # Same sweep in the other element type / layout / angle assignment (per-kernel times only,
@@ -344,6 +369,54 @@ def main():
             other_shapes[tag] = row
             del x, dy, y, dx, scr
             torch.cuda.empty_cache()
+
+    # ------------------------------------------------------------------ the reference's Table 5
+    # analysis/benchmark.py:19-67,84-104: one depthwise layer through the module and autograd,
+    # N=64, C=512, fp32, bias=False, stride 1, H=W in {14, 28, 56}, K in {7, 31}, one angle for all
+    # channels; per angle 10 warm-up iterations, then the mean wall-clock of `y = model(x);
+    # (y.mean() * 1024).backward()` between synchronisations, averaged over the eight angles.  x
+    # does not require a gradient there, so "fwd+bwd" is fprop + wgrad + the loss kernels.  The
+    # script passes its angles in degrees to a module that reads radians (and 66.75 for 67.5):
+    # "as_published" feeds those same numbers (non-canonical tap patterns: table-driven bodies),
+    # "canonical" the eight orientations k * 22.5 degrees the table's header means.  Published
+    # (README.md:318-327, one RTX 3090): 0.3/0.8, 0.9/2.6, 3.2/9.9 ms for K=7/31.
+    table5 = None
+    if args.table5_iters > 0 and not args.only:
+        from oriented1d_amd.dwoconv1d import DepthwiseOrientedConv1d as Conv
+
+        table5 = {"protocol": "N=64 C=512 f32 bias=False, fwd+bwd through the module as "
+                              "analysis/benchmark.py:19-67 times it, 10 warm-up + %d timed "
+                              "iterations per angle, mean over 8 angles, ms" % args.table5_iters,
+                  "published_rtx3090_ms": {"14": [0.3, 0.8], "28": [0.9, 2.6], "56": [3.2, 9.9]}}
+        published_angles = [0, 22.5, 45, 66.75, 90, 112.5, 135, 157.5]
+        torch.cuda.set_stream(torch.cuda.default_stream(dev))
+        for HW_ in (14, 28, 56):
+            xb = torch.randn(64, 512, HW_, HW_, device=dev)
+            row = {}
+            for K_ in (7, 31):
+                for tag, angles in (("as_published", published_angles),
+                                    ("canonical", [math.radians(a) for a in
+                                                   (0, 22.5, 45, 67.5, 90, 112.5, 135, 157.5)])):
+                    means = []
+                    for ang in angles:
+                        layer = Conv(512, 512, K_, angle=float(ang), padding=K_ // 2, stride=1,
+                                     bias=False, groups=512).to(dev)
+                        times = []
+                        for it in range(10 + args.table5_iters):
+                            torch.cuda.synchronize()
+                            t0 = time.perf_counter()
+                            (layer(xb).mean() * 1024).backward()
+                            for p_ in layer.parameters():
+                                p_.grad = None
+                            torch.cuda.synchronize()
+                            if it >= 10:
+                                times.append((time.perf_counter() - t0) * 1e3)
+                        means.append(sum(times) / len(times))
+                    row["K%d_%s" % (K_, tag)] = round(sum(means) / len(means), 3)
+            table5[str(HW_)] = row
+            del xb
+        torch.cuda.set_stream(stream)
+        torch.cuda.empty_cache()
 
     # ------------------------------------------------------------------ CPU baseline (oracle)
     cpu, cpu_all = None, None
@@ -528,15 +601,16 @@ def main():
                                "(C=96@56x56, 192@28x28, 384@14x14, 768@7x7), batch 64, K=31, "
                                "8 orientations %s, stride 1" % args.theta,
                    "layout": args.layout, "buffer_sets": nsets,
-                   "launch": "the faster of eager C-ABI calls and hipGraph replay of the step's 12 "
-                             "calls (one graph per buffer set); both are listed",
+                   "launch": "eager C-ABI calls on one stream (value, ms_per_step); the hipGraph "
+                             "replays of the same step are listed for information",
                    "ms_per_step_graph": round(main_res_graph, 4) if main_res_graph else None,
                    "ms_per_step_eager": round(main_res_eager, 4),
                    "ms_per_step_parallel_branches": (round(main_res_branches, 4)
                                                      if main_res_branches else None),
                    "algorithmic_bytes_per_step": step_bytes},
         "frac_hbm_peak": round(value / HBM_PEAK_GBS, 4),
-        "detail": detail, "roofline": roofline, "cpu_baseline": cpu,
+        "detail": detail, "roofline": roofline, "roofline_min": roofline_min, "cpu_baseline": cpu,
+        "table5": table5,
         "cpu_baseline_all_threads": cpu_all, "other_configs": others, "other_shapes_bf16": other_shapes,
         "convnext_t_1d": model_info, "training_configs": train_info,
     }

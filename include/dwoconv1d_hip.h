@@ -9,6 +9,18 @@
  * asynchronous on the stream passed in (the reference launches on the current stream,
  * models/dwoconv1d/kernels/kernels.cu:25).
  *
+ * First use.  The first launch of a kernel on a device queries its occupancy and sets its
+ * dynamic-LDS attribute, which a stream capture does not allow.  Call dwo_init() once per
+ * device (with that device current) before capturing calls into a graph; without it the set-up
+ * happens lazily inside the first call of each entry point on each shape class.  Each launching
+ * entry point clears the calling thread's HIP last-error state on entry, so the positive
+ * status it returns always belongs to its own launches.
+ *
+ * Tap blobs.  `taps` arguments are device copies of a blob built by dwo_build_taps for the
+ * same C and K as the call; the kernels index the blob with the call's C and K and cannot
+ * verify its header, so a blob of another size leads to out-of-range reads.  The caller checks
+ * the size (dwo_taps_bytes) before launching.
+ *
  * Operator definition (models/dwoconv1d_reference/kernels/kernels.cpp:36-52,71-90,111-126),
  * pad = K/2, P = ceil(H/stride), Q = ceil(W/stride):
  *   dh(s) = (int)(-sinf(theta_c) * (s - pad)),  dw(s) = (int)(cosf(theta_c) * (s - pad))
@@ -21,7 +33,11 @@
  * points read and write NHWC directly, which replaces the reference's transpose passes
  * (models/dwoconv1d/kernels/kernels.cu:56-68, nhwc_utils.h:46-110).
  * Element types: activations x, y, dy, dx are fp32, bf16 or fp16; weights, bias, dw and db
- * are always fp32 and all accumulation is fp32.
+ * are always passed as fp32 and all accumulation is fp32.  With 16-bit activations the
+ * row-direction orientations of the stride-1 plane kernels multiply through a two-element dot
+ * product whose operands are both in the activation type: there the weights are rounded to
+ * that type first (the reference holds the weights in the activation type throughout,
+ * models/dwoconv1d/kernels/kernels.cu:25); the error stays within the 16-bit tolerance.
  */
 #ifndef DWOCONV1D_HIP_H
 #define DWOCONV1D_HIP_H
@@ -58,6 +74,15 @@ int dwo_version(void);
 
 /* Human-readable text for a status returned by any entry point. */
 const char *dwo_status_string(int status);
+
+/*
+ * One-time set-up of every kernel on the current device (occupancy queries, dynamic-LDS
+ * attributes), so that later calls only launch kernels and can be captured into a graph.
+ * Replaces nothing the reference's extension exports: there the set-up is the JIT build plus
+ * the cudaFuncSetAttribute of every launcher call (models/dwoconv1d/kernels/kernels.h:520-531).
+ * Idempotent and thread-safe; call once per device with that device current.
+ */
+int dwo_init(void);
 
 /*
  * Host-side tap table.  Replaces the per-thread sincosf + truncation of the reference

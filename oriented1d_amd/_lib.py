@@ -15,6 +15,7 @@ _vp, _i, _sz = ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t
 SIGNATURES = {
     "dwo_version": (_i, []),
     "dwo_status_string": (ctypes.c_char_p, [_i]),
+    "dwo_init": (_i, []),
     "dwo_taps_bytes": (_sz, [_i, _i]),
     "dwo_build_taps": (_i, [_vp, _i, _i, _vp]),
     "dwo_taps_get": (_i, [_vp, _i, _i, ctypes.POINTER(_i), ctypes.POINTER(_i)]),
@@ -46,6 +47,22 @@ def load():
         fn = getattr(lib, name)
         fn.restype, fn.argtypes = res, args
     _lib = lib
+    return lib
+
+
+_ready = set()
+
+
+def ready(device):
+    """The loaded library with its kernels set up on ``device`` (a torch CUDA device): the first
+    use on a device runs ``dwo_init`` there, so no later call does anything but launch kernels."""
+    lib = load()
+    if device.index not in _ready:
+        import torch
+
+        with torch.cuda.device(device):
+            check(lib.dwo_init(), "dwo_init")
+        _ready.add(device.index)
     return lib
 
 

@@ -1,5 +1,7 @@
 // C ABI of libdwoconv1d_hip.so: argument validation, host-side tap table, kernel selection
-// and launch.  No device allocation, no retained pointers, no global mutable state.
+// and launch.  No device allocation and no retained caller pointers; the only state is what
+// dwo_init caches per device (occupancy figures, kernel attributes, the address of the static
+// wgrad scratch).
 #include <math.h>
 #include <stdlib.h>
 #include <string.h>
@@ -40,6 +42,11 @@ int launch_status() {
     hipError_t e = hipGetLastError();
     return e == hipSuccess ? DWO_OK : (int)e;
 }
+
+// The launchers report hipGetLastError() after their launch; an error left behind on this
+// thread by unrelated earlier work must not be returned as this call's status, so every
+// launching entry point starts by clearing it.
+void begin_call() { (void)hipGetLastError(); }
 
 struct WgradSplit {
     int blocks_x, G, per_slice;
@@ -312,11 +319,62 @@ int pointwise_fprop_t(const void *x, const float *pw_w, const float *pw_b, const
     }
 }
 
+int wgrad_dispatch(const void *dy, const void *x, const void *taps, float *dw, float *db,
+                   void *scratch, int N, int C, int H, int W, int K, int stride, int dtype,
+                   int layout, hipStream_t st) {
+    const ConvDims d = make_dims(N, C, H, W, K, stride);
+    begin_call();
+    switch (dtype) {
+        case DWO_F32: return wgrad_t<float>(dy, x, taps, dw, db, scratch, d, layout, st);
+        case DWO_BF16: return wgrad_t<bf16_t>(dy, x, taps, dw, db, scratch, d, layout, st);
+        default: return wgrad_t<f16_t>(dy, x, taps, dw, db, scratch, d, layout, st);
+    }
+}
+
+// One-time set-up of every kernel on the current device (see per_device_once): the launchers
+// are called with an empty batch, which stops them after their set-up.
+template <typename T>
+int init_type() {
+    int rc = 0, ng = 0;
+#define DWO_PREP(K_, H_, W_)                                                                      \
+    rc |= launch_plane_conv<T, K_, H_, W_>(OP_FPROP, nullptr, nullptr, nullptr, nullptr, nullptr, \
+                                           0, 1, nullptr);                                        \
+    rc |= launch_plane_wgrad<T, K_, H_, W_>(nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, \
+                                            0, 1, &ng, nullptr);                                  \
+    rc |= launch_nhwc_plane_conv<T, K_, H_, W_>(OP_FPROP, nullptr, nullptr, nullptr, nullptr,     \
+                                                nullptr, 0, kSliceCh, nullptr);                   \
+    rc |= launch_nhwc_plane_wgrad<T, K_, H_, W_>(nullptr, nullptr, nullptr, nullptr, nullptr,     \
+                                                 nullptr, 0, kSliceCh, &ng, nullptr);
+    DWO_PLANE_SHAPES(DWO_PREP)
+#undef DWO_PREP
+    ConvDims d = make_dims(1, kSliceCh, 8, 8, 7, 2);
+    d.N = 0;
+    rc |= launch_nchw_tile_fprop<T>(nullptr, nullptr, nullptr, nullptr, nullptr, d, 0, nullptr);
+    rc |= launch_nhwc_tile_fprop<T>(nullptr, nullptr, nullptr, nullptr, nullptr, d, 0, nullptr);
+    rc |= launch_tile_dgrad_strided<T>(nullptr, nullptr, nullptr, nullptr, d, true, nullptr);
+    rc |= launch_tile_dgrad_strided<T>(nullptr, nullptr, nullptr, nullptr, d, false, nullptr);
+    rc |= launch_tile_wgrad<T>(nullptr, nullptr, nullptr, nullptr, &ng, d, true, nullptr);
+    rc |= launch_tile_wgrad<T>(nullptr, nullptr, nullptr, nullptr, &ng, d, false, nullptr);
+    for (int cin = 1; cin <= 4; cin++)
+        rc |= pointwise_fprop_t<T>(nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr,
+                                   cin, d, nullptr);
+    return rc;
+}
+
 }  // namespace
 
 extern "C" {
 
-int dwo_version(void) { return 100; }
+int dwo_init(void) {
+    begin_call();
+    // (the set-up calls leave their own failures in the runtime's last-error slot)
+    (void)init_type<float>();
+    (void)init_type<bf16_t>();
+    (void)init_type<f16_t>();
+    return launch_status();
+}
+
+int dwo_version(void) { return 200; }
 
 const char *dwo_status_string(int status) {
     switch (status) {
@@ -415,6 +473,7 @@ int dwo_fprop(const void *x, const float *w, const float *bias, const void *taps
     if (!x || !w || !taps || !y) return DWO_ERR_NULL_POINTER;
     const ConvDims d = make_dims(N, C, H, W, K, stride);
     hipStream_t st = (hipStream_t)stream;
+    begin_call();
     switch (dtype) {
         case DWO_F32: return fprop_t<float>(x, w, bias, taps, y, d, layout, st);
         case DWO_BF16: return fprop_t<bf16_t>(x, w, bias, taps, y, d, layout, st);
@@ -429,6 +488,7 @@ int dwo_dgrad(const void *dy, const float *w, const void *taps, void *dx, int N,
     if (!dy || !w || !taps || !dx) return DWO_ERR_NULL_POINTER;
     const ConvDims d = make_dims(N, C, H, W, K, stride);
     hipStream_t st = (hipStream_t)stream;
+    begin_call();
     switch (dtype) {
         case DWO_F32: return dgrad_t<float>(dy, w, taps, dx, d, layout, st);
         case DWO_BF16: return dgrad_t<bf16_t>(dy, w, taps, dx, d, layout, st);
@@ -451,13 +511,8 @@ int dwo_wgrad(const void *dy, const void *x, const void *taps, float *dw, float 
     if (!dy || !x || !taps || !dw || !scratch) return DWO_ERR_NULL_POINTER;
     if (scratch_bytes < dwo_wgrad_scratch_bytes(N, C, H, W, K, stride, dtype, layout))
         return DWO_ERR_SCRATCH_TOO_SMALL;
-    const ConvDims d = make_dims(N, C, H, W, K, stride);
-    hipStream_t st = (hipStream_t)stream;
-    switch (dtype) {
-        case DWO_F32: return wgrad_t<float>(dy, x, taps, dw, db, scratch, d, layout, st);
-        case DWO_BF16: return wgrad_t<bf16_t>(dy, x, taps, dw, db, scratch, d, layout, st);
-        default: return wgrad_t<f16_t>(dy, x, taps, dw, db, scratch, d, layout, st);
-    }
+    return wgrad_dispatch(dy, x, taps, dw, db, scratch, N, C, H, W, K, stride, dtype, layout,
+                          (hipStream_t)stream);
 }
 
 int dwo_pointwise_fprop_nhwc(const void *x, const float *pw_w, const float *pw_b, const float *w,
@@ -469,6 +524,7 @@ int dwo_pointwise_fprop_nhwc(const void *x, const float *pw_w, const float *pw_b
     if (Cin < 1 || Cin > 4 || C % kSliceCh != 0) return DWO_ERR_BAD_SHAPE;
     const ConvDims d = make_dims(N, C, H, W, K, stride);
     hipStream_t st = (hipStream_t)stream;
+    begin_call();
     switch (dtype) {
         case DWO_F32: return pointwise_fprop_t<float>(x, pw_w, pw_b, w, bias, taps, y, Cin, d, st);
         case DWO_BF16: return pointwise_fprop_t<bf16_t>(x, pw_w, pw_b, w, bias, taps, y, Cin, d, st);
@@ -481,6 +537,7 @@ int dwo_layernorm_nhwc(const void *x, const float *gamma, const float *beta, voi
     if (!x || !gamma || !beta || !out) return DWO_ERR_NULL_POINTER;
     if (rows < 1 || C < 2 || (C & 1) || C > kFusedMaxC) return DWO_ERR_BAD_SHAPE;
     hipStream_t st = (hipStream_t)stream;
+    begin_call();
     switch (dtype) {
         case DWO_F32: return launch_layernorm_nhwc<float>(x, gamma, beta, out, (long)rows, C, eps, gelu, st);
         case DWO_BF16: return launch_layernorm_nhwc<bf16_t>(x, gamma, beta, out, (long)rows, C, eps, gelu, st);
@@ -496,6 +553,7 @@ int dwo_nchw_layernorm_nhwc(const void *x, const float *gamma, const float *beta
         (long)H * W > 0x7fffffffL / C)
         return DWO_ERR_BAD_SHAPE;
     hipStream_t st = (hipStream_t)stream;
+    begin_call();
     switch (dtype) {
         case DWO_F32: return launch_nchw_layernorm_nhwc<float>(x, gamma, beta, out, N, C, H * W, eps, st);
         case DWO_BF16: return launch_nchw_layernorm_nhwc<bf16_t>(x, gamma, beta, out, N, C, H * W, eps, st);
@@ -510,6 +568,7 @@ int dwo_nhwc_scale_add_nchw(const void *y, const float *scale, const void *res, 
     if (N < 1 || N > 65535 || H < 1 || W < 1 || C < 2 || (C & 1) || (long)H * W > 0x7fffffffL / C)
         return DWO_ERR_BAD_SHAPE;
     hipStream_t st = (hipStream_t)stream;
+    begin_call();
     switch (dtype) {
         case DWO_F32: return launch_nhwc_scale_add_nchw<float>(y, scale, res, out, N, C, H * W, st);
         case DWO_BF16: return launch_nhwc_scale_add_nchw<bf16_t>(y, scale, res, out, N, C, H * W, st);

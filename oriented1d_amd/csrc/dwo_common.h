@@ -107,6 +107,23 @@ void allow_large_lds(Kern kern, size_t lds) {
                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
 }
 
+// One-time set-up of a kernel on a device (dynamic-LDS attribute, occupancy query): `make()` runs
+// once per device with that device current and its non-zero result is kept in cache[device].
+// Launchers called with an empty batch (N = 0) stop right after it, which is how dwo_init
+// prepares every kernel ahead of a stream capture.
+constexpr int kMaxDevices = 64;
+template <class F>
+inline int per_device_once(int *cache, F make) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return make();
+    int v = __atomic_load_n(&cache[dev], __ATOMIC_ACQUIRE);
+    if (v == 0) {
+        v = make();  // idempotent: two threads racing here compute the same value
+        __atomic_store_n(&cache[dev], v, __ATOMIC_RELEASE);
+    }
+    return v;
+}
+
 struct ConvDims {
     int N, C, H, W, P, Q, K, stride, shift;  // shift = log2(stride)
 };

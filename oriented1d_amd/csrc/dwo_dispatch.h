@@ -10,11 +10,13 @@
 
 // X(K, H, W): kernel size and plane extents with compile-time kernels (stride 1): the ConvNeXt
 // stage extents at 224 x 224 input for K = 31 (1D blocks, second conv of 1D++ blocks) and K = 15
-// (first conv of 1D++ blocks)
+// (first conv of 1D++ blocks), and K = 7 at the three extents of the reference's own
+// micro-benchmark (analysis/benchmark.py:84-104)
 #ifndef DWO_PLANE_SHAPES
 #define DWO_PLANE_SHAPES(X)                                   \
     X(31, 56, 56) X(31, 28, 28) X(31, 14, 14) X(31, 7, 7)     \
-    X(15, 56, 56) X(15, 28, 28) X(15, 14, 14) X(15, 7, 7)
+    X(15, 56, 56) X(15, 28, 28) X(15, 14, 14) X(15, 7, 7)     \
+    X(7, 56, 56) X(7, 28, 28) X(7, 14, 14)
 #endif
 
 namespace dwo {

@@ -304,11 +304,13 @@ int launch_nhwc_plane_conv(int op, const void *src, const float *w, const float 
                            const void *taps, void *dst, int N, int C, hipStream_t st) {
     constexpr int NT = NhwcTile<H, W>::NT, PBI = NhwcTile<H, W>::PBI;
     const size_t lds = nhwc_plane_lds_bytes<K, H, W>();
-    static const int slots = [&] {
+    static int cache[kMaxDevices];
+    const int slots = per_device_once(cache, [&] {
         allow_large_lds(nhwc_plane_kernel<OP_FPROP, T, K, H, W>, lds);
         allow_large_lds(nhwc_plane_kernel<OP_DGRAD, T, K, H, W>, lds);
         return resident_slots(nhwc_plane_kernel<OP_FPROP, T, K, H, W>, NT, lds);
-    }();
+    });
+    if (N == 0) return 0;  // set-up only
     const int nslices = C / kSliceCh;
     const int groups = plane_groups(N, nslices, PBI, slots);
     const dim3 grid(nslices * groups), block(NT);
@@ -641,10 +643,12 @@ int launch_nhwc_plane_wgrad(const void *x, const void *dy, const void *taps, flo
                             float *db, int N, int C, int *groups_out, hipStream_t st) {
     constexpr int NT = NhwcTile<H, W>::NT, PBI = NhwcTile<H, W>::PBI;
     const size_t lds = nhwc_plane_wgrad_lds_bytes<K, H, W>();
-    static const int slots = [&] {
+    static int cache[kMaxDevices];
+    const int slots = per_device_once(cache, [&] {
         allow_large_lds(nhwc_plane_wgrad_kernel<T, K, H, W>, lds);
         return resident_slots(nhwc_plane_wgrad_kernel<T, K, H, W>, NT, lds);
-    }();
+    });
+    if (N == 0) return 0;  // set-up only
     const int nslices = C / kSliceCh;
     const int groups = plane_groups(N, nslices, PBI, slots);
     *groups_out = groups;

@@ -447,11 +447,12 @@ template <typename T, class Src>
 int launch_nhwc_tile(const typename Src::Params &sp, const float *w, const float *bias,
                      const void *taps, void *y, const ConvDims &d, int flip, hipStream_t st) {
     const size_t lds = nhwc_tile_lds_bytes<T>();
-    static const bool once = [&] {
+    static int cache[kMaxDevices];
+    per_device_once(cache, [&] {
         allow_large_lds(nhwc_tile_fprop_kernel<T, Src>, lds);
-        return true;
-    }();
-    (void)once;
+        return 1;
+    });
+    if (d.N == 0) return 0;  // set-up only
     const int nslices = (d.C + kSliceCh - 1) / kSliceCh;
     const int band_rows = tile_band_rows(d.N, d.P, nslices);
     const int nbands = (d.P + band_rows - 1) / band_rows;
@@ -693,11 +694,12 @@ template <typename T, class Src>
 int launch_tile_dgrad_strided_src(const void *dy, const float *w, const void *taps, void *dx,
                                   const ConvDims &d, hipStream_t st) {
     const size_t lds = tile_dgrad_lds_bytes<T>();
-    static const bool once = [&] {
+    static int cache[kMaxDevices];
+    per_device_once(cache, [&] {
         allow_large_lds(tile_dgrad_strided_kernel<T, Src>, lds);
-        return true;
-    }();
-    (void)once;
+        return 1;
+    });
+    if (d.N == 0) return 0;  // set-up only
     const int nslices = (d.C + kSliceCh - 1) / kSliceCh;
     const int band_rows = tile_band_rows(d.N, d.H, nslices);
     const int nbands = (d.H + band_rows - 1) / band_rows;
@@ -914,11 +916,12 @@ template <typename T, class Src>
 int launch_tile_wgrad_src(const void *x, const void *dy, const void *taps, float *part, int *groups,
                           const ConvDims &d, hipStream_t st) {
     const size_t lds = tile_wgrad_lds_bytes<T>();
-    static const bool once = [&] {
+    static int cache[kMaxDevices];
+    per_device_once(cache, [&] {
         allow_large_lds(tile_wgrad_kernel<T, Src>, lds);
-        return true;
-    }();
-    (void)once;
+        return 1;
+    });
+    if (d.N == 0) return 0;  // set-up only
     int band_rows, nbands;
     const int G = tile_wgrad_groups(d, &band_rows, &nbands);
     *groups = G;

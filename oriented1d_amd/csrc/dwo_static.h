@@ -905,7 +905,10 @@ int launch_plane_conv(int op, const void *src, const float *w, const float *bias
                       void *dst, int N, int C, hipStream_t st) {
     constexpr int NT = Tile<H, W>::NT;
     const size_t lds = plane_kernel_lds_bytes<T, K, H, W>();
-    static const int slots_f = resident_slots(plane_kernel<OP_FPROP, T, K, H, W>, NT, lds);
+    static int cache[kMaxDevices];
+    const int slots_f = per_device_once(
+        cache, [&] { return resident_slots(plane_kernel<OP_FPROP, T, K, H, W>, NT, lds); });
+    if (N == 0) return 0;  // set-up only
     const int groups = plane_groups(N, C, Tile<H, W>::PB, slots_f);
     const dim3 grid(C * groups), block(NT);
     if (op == OP_FPROP)
@@ -925,7 +928,10 @@ int launch_plane_wgrad(const void *x, const void *dy, const void *taps, float *p
                        float *db, int N, int C, int *groups_out, hipStream_t st) {
     constexpr int NT = Tile<H, W>::NT;
     const size_t lds = plane_wgrad_lds_bytes<K, H, W>();
-    static const int slots = resident_slots(plane_wgrad_kernel<T, K, H, W>, NT, lds);
+    static int cache[kMaxDevices];
+    const int slots = per_device_once(
+        cache, [&] { return resident_slots(plane_wgrad_kernel<T, K, H, W>, NT, lds); });
+    if (N == 0) return 0;  // set-up only
     const int groups = plane_groups(N, C, Tile<H, W>::PB, slots);
     *groups_out = groups;
     plane_wgrad_kernel<T, K, H, W><<<dim3(C * groups), dim3(NT), lds, st>>>(

@@ -79,18 +79,37 @@ def taps_to_numpy(blob, C, K):
 
 
 class _TapCache:
-    """Device tap table of one theta tensor, rebuilt when theta is modified or moved."""
+    """Device tap tables, one per (theta tensor, device, C, K), rebuilt when theta is modified
+    or moved.  A module owns one (a single entry in practice); the five-function tuple of
+    ``oriented_dwconv1d_get_module_from_params`` owns one that may serve several layers, so the
+    few most recent tables are kept."""
+
+    KEEP = 8
 
     def __init__(self):
-        self.key = None
-        self.dev = None
+        self.entries = {}  # (id(theta), device, C, K) -> (state key, weak ref, device blob)
 
     def get(self, theta, C, K, device):
-        key = (theta.data_ptr(), theta._version, str(device), C, K)
-        if key != self.key:
-            self.dev = build_taps(theta, C, K).to(device)
-            self.key = key
-        return self.dev
+        slot = (id(theta), str(device), C, K)
+        state = (theta.data_ptr(), theta._version)
+        hit = self.entries.get(slot)
+        if hit is None or hit[0] != state or hit[1]() is not theta:
+            if len(self.entries) >= self.KEEP:
+                self.entries.pop(next(iter(self.entries)))
+            blob = build_taps(theta, C, K).to(device)
+            hit = (state, weakref.ref(theta), blob)
+            self.entries[slot] = hit
+        return hit[2]
+
+
+def _check_taps(taps, C, K):
+    """The device kernels index the tap blob with the C and K they are launched with and cannot
+    see its header without a device read, so the size is checked here: a blob of
+    ``dwo_taps_bytes(C, K)`` bytes keeps every table read in range."""
+    want = _lib.load().dwo_taps_bytes(C, K)
+    if taps.dtype != torch.uint8 or taps.numel() != want:
+        raise RuntimeError("tap table does not match C=%d, K=%d (%d bytes, expected %d)"
+                           % (C, K, taps.numel(), want))
 
 
 def _dims(x, nhwc):
@@ -132,11 +151,12 @@ def f32_copy(p):
 
 def fprop(x, w, taps, stride=1, bias=None, nhwc=False):
     """y = fprop(x, w, theta) (+ bias).  x: [N,C,H,W] or [N,H,W,C]; w: [C,1,1,K]."""
-    lib = _lib.load()
     _check_activation(x, "x")
+    lib = _lib.ready(x.device)
     N, C, H, W = _dims(x, nhwc)
     w2 = _w2d(w, C)
     K = w2.shape[1]
+    _check_taps(taps, C, K)
     b = f32_copy(bias) if bias is not None else None
     y = torch.empty(_out_shape(N, C, H, W, stride, nhwc), dtype=x.dtype, device=x.device)
     _lib.check(lib.dwo_fprop(_ptr(x), _ptr(w2), _ptr(b), _ptr(taps), _ptr(y), N, C, H, W, K,
@@ -146,14 +166,15 @@ def fprop(x, w, taps, stride=1, bias=None, nhwc=False):
 
 def dgrad(dy, w, taps, in_hw, stride=1, nhwc=False):
     """dx = dgrad(dy, w, theta); ``in_hw`` is the (H, W) of the forward input."""
-    lib = _lib.load()
     _check_activation(dy, "dy")
+    lib = _lib.ready(dy.device)
     H, W = in_hw
     N, C, P, Q = _dims(dy, nhwc)
     if (P, Q) != (-(-H // stride), -(-W // stride)):
         raise RuntimeError("dy extent does not match the input extent and stride")
     w2 = _w2d(w, C)
     K = w2.shape[1]
+    _check_taps(taps, C, K)
     dx = torch.empty((N, H, W, C) if nhwc else (N, C, H, W), dtype=dy.dtype, device=dy.device)
     _lib.check(lib.dwo_dgrad(_ptr(dy), _ptr(w2), _ptr(taps), _ptr(dx), N, C, H, W, K, stride,
                              _DTYPES[dy.dtype], int(nhwc), _stream(dy)), "dwo_dgrad")
@@ -162,14 +183,15 @@ def dgrad(dy, w, taps, in_hw, stride=1, nhwc=False):
 
 def wgrad(dy, x, taps, K, stride=1, nhwc=False, with_bias=False):
     """(dw [C,1,1,K] fp32, db [C] fp32 or None) = wgrad(dy, x, theta)."""
-    lib = _lib.load()
     _check_activation(dy, "dy")
     _check_activation(x, "x")
+    lib = _lib.ready(x.device)
     if dy.dtype != x.dtype:
         raise RuntimeError("dy and x must have the same dtype")
     N, C, H, W = _dims(x, nhwc)
     if tuple(dy.shape) != _out_shape(N, C, H, W, stride, nhwc):
         raise RuntimeError("dy extent does not match the input extent and stride")
+    _check_taps(taps, C, K)
     dt, lay = _DTYPES[x.dtype], int(nhwc)
     nbytes = lib.dwo_wgrad_scratch_bytes(N, C, H, W, K, stride, dt, lay)
     scratch = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=x.device)
@@ -180,19 +202,53 @@ def wgrad(dy, x, taps, K, stride=1, nhwc=False, with_bias=False):
     return dw, db
 
 
+class KernelTuple(tuple):
+    """The reference's five-function tuple ``(fprop, dgrad, wgrad, nhwc_to_nchw, nchw_to_nhwc)``
+    (models/dwoconv1d/dwoconv1d.py:72-80) plus what the native path needs to run without the
+    transposes: kernel size, stride, a tap-table cache, and whether extents that the stride does
+    not divide are accepted."""
+
+    def __new__(cls, functions, kernel_size, stride, arbitrary_size):
+        self = super().__new__(cls, functions)
+        self.kernel_size, self.stride = kernel_size, stride
+        self.arbitrary_size = arbitrary_size
+        self.taps = _TapCache()
+        return self
+
+    def __reduce__(self):
+        # copies (copy.deepcopy of a model, e.g. for an averaged twin) and pickles are rebuilt
+        # from the parameters; the tap cache starts empty
+        return (oriented_dwconv1d_get_module_from_params,
+                ("float", self.kernel_size, self.stride, self.kernel_size // 2,
+                 4 if self.arbitrary_size else 1))
+
+
 class _DepthwiseOrientedConv1d(torch.autograd.Function):
     """Autograd contract of models/dwoconv1d/dwoconv1d.py:18-69.
 
-    ``apply(x, w, theta, bias, module, nhwc, resid)``; ``module`` is the owning
-    ``DepthwiseOrientedConv1d`` (the reference passes its tuple of compiled functions in
-    this slot).  backward returns (dx, dw, None, db, None, None, None): theta never
+    ``apply(x, w, theta, bias, module, nhwc, resid)``.  ``module`` is what the reference passes
+    in this slot, the tuple returned by ``oriented_dwconv1d_get_module_from_params`` (a
+    ``KernelTuple`` here): the convolution then runs natively in the tensor's layout with the
+    bias fused.  Any other 5-tuple of callables is driven exactly as the reference drives its
+    own (transposes, separate bias add, ``dy.sum``), and the owning ``DepthwiseOrientedConv1d``
+    is accepted as well.  backward returns (dx, dw, None, db, None, None, None): theta never
     receives a gradient (dwoconv1d.py:64)."""
 
     @staticmethod
     def forward(ctx, x, w, theta, bias, module, nhwc=False, resid=None):
-        stride = module.stride[0]
+        ctx.set_materialize_grads(False)
+        if isinstance(module, DepthwiseOrientedConv1d):
+            module = module.module_fp32_large if module.arbitrary_size else module.module_fp32
+        ctx.plain = None
+        if not isinstance(module, KernelTuple):
+            return _DepthwiseOrientedConv1d._forward_plain(ctx, x, w, theta, bias, module, nhwc,
+                                                           resid)
+        stride = module.stride
         C = w.shape[0]
         K = w.shape[-1]
+        if K != module.kernel_size:
+            raise RuntimeError("weight has %d taps, the kernel tuple was made for %d"
+                               % (K, module.kernel_size))
         w_eff = f32_copy(w)
         if resid is not None:
             w_eff = w_eff + resid.to(w_eff)
@@ -204,9 +260,8 @@ class _DepthwiseOrientedConv1d(torch.autograd.Function):
         if not module.arbitrary_size and (H % stride != 0 or W % stride != 0):
             # models/dwoconv1d/kernels/kernels.cu:20
             raise RuntimeError("Invalid input size: H,W not divisible by stride")
-        taps = module._taps.get(theta, C, K, x.device)
+        taps = module.taps.get(theta, C, K, x.device)
 
-        ctx.set_materialize_grads(False)
         ctx.stride, ctx.nhwc, ctx.K = stride, nhwc, K
         ctx.with_bias = bias is not None
         ctx.w_dtype = w.dtype
@@ -215,9 +270,42 @@ class _DepthwiseOrientedConv1d(torch.autograd.Function):
         return fprop(x, w_eff, taps, stride, bias=bias, nhwc=nhwc)
 
     @staticmethod
+    def _forward_plain(ctx, x, w, theta, bias, module, nhwc, resid):
+        # models/dwoconv1d/dwoconv1d.py:21-38, for a caller's own five functions
+        f, _, _, nhwc_to_nchw, nchw_to_nhwc = module
+        if resid is not None:
+            w = w + resid
+        x = x.contiguous()
+        if nhwc:
+            x = nhwc_to_nchw(x)
+        ctx.plain, ctx.nhwc = module, nhwc
+        ctx.save_for_backward(x, w, theta, bias)
+        y = f(x, w, theta)
+        if bias is not None:
+            y = y + bias.to(y).view(1, -1, 1, 1)
+        return nchw_to_nhwc(y) if nhwc else y
+
+    @staticmethod
     def backward(ctx, dy):
         if dy is None:
             return None, None, None, None, None, None, None
+        if ctx.plain is not None:
+            # models/dwoconv1d/dwoconv1d.py:45-69
+            _, d, g, nhwc_to_nchw, nchw_to_nhwc = ctx.plain
+            x, w, theta, bias = ctx.saved_tensors
+            dy = dy.contiguous()
+            if ctx.nhwc:
+                dy = nhwc_to_nchw(dy)
+            dx = dw = db = None
+            if ctx.needs_input_grad[0]:
+                dx = d(dy, w, theta)
+                if ctx.nhwc:
+                    dx = nchw_to_nhwc(dx)
+            if ctx.needs_input_grad[1]:
+                dw = g(dy, x, theta)
+            if bias is not None and ctx.needs_input_grad[3]:
+                db = dy.sum(dim=[0, 2, 3])
+            return dx, dw, None, db, None, None, None
         x, w_eff, taps = ctx.saved_tensors
         dy = dy.contiguous()
         if dy.dtype != x.dtype:
@@ -241,24 +329,28 @@ class _DepthwiseOrientedConv1d(torch.autograd.Function):
 def oriented_dwconv1d_get_module_from_params(ftype, kernel_size, stride, pad, Sb=None):
     """Five-function tuple in the reference's order (models/dwoconv1d/dwoconv1d.py:72-80):
     (fprop(x,w,theta), dgrad(dy,w,theta), wgrad(dy,x,theta), nhwc_to_nchw, nchw_to_nhwc),
-    all on NCHW tensors.  ``ftype``, ``pad`` and ``Sb`` are accepted for signature
-    compatibility: there is nothing to compile per configuration, pad is always
-    ``kernel_size // 2`` and the kernels need no filter partitioning."""
+    all on contiguous NCHW tensors; the result goes into slot 5 of
+    ``_DepthwiseOrientedConv1d.apply`` as in the reference (dwoconv1d.py:189-198).
+    ``ftype`` and ``pad`` are accepted for signature compatibility: there is nothing to compile
+    per configuration and pad is always ``kernel_size // 2``.  The kernels need no filter
+    partitioning; ``Sb=4`` is how the reference asks for its arbitrary-size variant
+    (dwoconv1d.py:150-152), so such a tuple accepts extents the stride does not divide
+    (output ceil(H/stride)), any other rejects them as kernels.cu:20 does."""
     K = int(kernel_size)
     stride = int(stride)
-
-    def _taps(theta, C, dev):
-        return build_taps(theta, C, K).to(dev)
+    arbitrary = Sb is not None and int(Sb) > 1
 
     def f(x, w, theta):
-        return fprop(x, w, _taps(theta, x.shape[1], x.device), stride)
+        if not arbitrary and (x.shape[2] % stride != 0 or x.shape[3] % stride != 0):
+            raise RuntimeError("Invalid input size: H,W not divisible by stride")
+        return fprop(x, w, kt.taps.get(theta, x.shape[1], K, x.device), stride)
 
     def d(dy, w, theta):
         hw = (dy.shape[2] * stride, dy.shape[3] * stride)
-        return dgrad(dy, w, _taps(theta, dy.shape[1], dy.device), hw, stride)
+        return dgrad(dy, w, kt.taps.get(theta, dy.shape[1], K, dy.device), hw, stride)
 
     def g(dy, x, theta):
-        return wgrad(dy, x, _taps(theta, x.shape[1], x.device), K, stride)[0].to(x.dtype)
+        return wgrad(dy, x, kt.taps.get(theta, x.shape[1], K, x.device), K, stride)[0].to(x.dtype)
 
     def nhwc_to_nchw(x):
         return x.permute(0, 3, 1, 2).contiguous()
@@ -266,7 +358,8 @@ def oriented_dwconv1d_get_module_from_params(ftype, kernel_size, stride, pad, Sb
     def nchw_to_nhwc(x):
         return x.permute(0, 2, 3, 1).contiguous()
 
-    return f, d, g, nhwc_to_nchw, nchw_to_nhwc
+    kt = KernelTuple((f, d, g, nhwc_to_nchw, nchw_to_nhwc), K, stride, arbitrary)
+    return kt
 
 
 class DepthwiseOrientedConv1d(nn.Conv2d):
@@ -322,7 +415,12 @@ class DepthwiseOrientedConv1d(nn.Conv2d):
             self.register_buffer("resid", onehot, persistent=False)
         else:
             self.resid = None
-        self._taps = _TapCache()
+        # models/dwoconv1d/dwoconv1d.py:144-152: the tuples forward() hands to apply()
+        self.module_fp32 = oriented_dwconv1d_get_module_from_params(
+            "float", kernel_size, self.stride[0], pad, Sb=1)
+        if arbitrary_size:
+            self.module_fp32_large = oriented_dwconv1d_get_module_from_params(
+                "float", kernel_size, self.stride[0], pad, Sb=4)
 
     def _apply(self, fn, recurse=True):
         """``.to()/.half()/.bfloat16()/.cuda()`` move and cast weight and bias, but the angles stay
@@ -335,11 +433,22 @@ class DepthwiseOrientedConv1d(nn.Conv2d):
             self.theta.data = theta.to(self.theta.device)
         return self
 
+    @property
+    def _taps(self):
+        """Tap-table cache of the tuple forward() uses."""
+        return (self.module_fp32_large if self.arbitrary_size else self.module_fp32).taps
+
     def forward_safe(self, x):
-        """Arbitrary H, W (reference: dwoconv1d.py:154-187); handled natively."""
-        return self.forward(x)
+        """Arbitrary H, W (reference: dwoconv1d.py:154-187): no padding to a power of two, no
+        crop and no permuted copies; the kernels produce ceil(H/stride) x ceil(W/stride)
+        outputs in the tensor's own layout, the values that path returns."""
+        return _DepthwiseOrientedConv1d.apply(
+            x, self.weight, self.theta, self.bias, self.module_fp32_large, self.nhwc, self.resid
+        )
 
     def forward(self, x):
+        if self.arbitrary_size:  # the reference rebinds forward to forward_safe (:148-149)
+            return self.forward_safe(x)
         return _DepthwiseOrientedConv1d.apply(
-            x, self.weight, self.theta, self.bias, self, self.nhwc, self.resid
+            x, self.weight, self.theta, self.bias, self.module_fp32, self.nhwc, self.resid
         )

@@ -100,7 +100,7 @@ def pointwise_dwconv_nhwc(x, linear, conv):
     pw_b = _f32(linear.bias) if linear.bias is not None else None
     w2 = w.reshape(C, K)
     cb = _f32(conv.bias) if conv.bias is not None else None
-    _lib.check(_lib.load().dwo_pointwise_fprop_nhwc(
+    _lib.check(_lib.ready(x.device).dwo_pointwise_fprop_nhwc(
         _ptr(x), _ptr(pw_w), _ptr(pw_b), _ptr(w2), _ptr(cb), _ptr(taps), _ptr(y), N, Cin, C, H, W,
         K, stride, _DTYPES[x.dtype], _stream(x)), "dwo_pointwise_fprop_nhwc")
     return y

@@ -156,3 +156,46 @@ def test_angles_stay_fp32_under_module_casts():
     dh0, dw0 = op.taps_to_numpy(op.build_taps(before, C, K), C, K)
     dh1, dw1 = op.taps_to_numpy(op.build_taps(rounded_theta, C, K), C, K)
     assert (dh0 != dh1).any() or (dw0 != dw1).any()
+
+
+def test_backward_without_upstream_gradient_returns_nones():
+    """dwoconv1d.py:42-43: an undefined upstream gradient short-circuits to seven Nones (the
+    Function does not materialise gradients, :28)."""
+    out = op._DepthwiseOrientedConv1d.backward(object(), None)
+    assert out == (None,) * 7
+
+
+def test_specialized_import_name_and_tuple_contract():
+    """models/convnext.py:16-23 imports the module under either name; the tuple in slot 5 of
+    apply() carries what the native path needs (dwoconv1d.py:72-80,144-152)."""
+    import copy
+    import pickle
+
+    import dwoconv1d_specialized as spec
+    assert spec.DepthwiseOrientedConv1d is op.DepthwiseOrientedConv1d
+    m = op.DepthwiseOrientedConv1d(8, 8, 7, groups=8, stride=2, angle=0.3, arbitrary_size=True)
+    assert isinstance(m.module_fp32, op.KernelTuple) and len(m.module_fp32) == 5
+    assert (m.module_fp32.kernel_size, m.module_fp32.stride, m.module_fp32.arbitrary_size) == (7, 2, False)
+    assert m.module_fp32_large.arbitrary_size
+    assert m._taps is m.module_fp32_large.taps
+    assert not hasattr(op.DepthwiseOrientedConv1d(8, 8, 7, groups=8), "module_fp32_large")
+    for twin in (copy.deepcopy(m), pickle.loads(pickle.dumps(m))):
+        assert isinstance(twin.module_fp32, op.KernelTuple) and twin.module_fp32 is not m.module_fp32
+        assert twin.module_fp32.stride == 2 and twin.module_fp32_large.arbitrary_size
+        assert list(twin.state_dict()) == ["weight", "bias", "theta"]
+    # CPU tensors are refused by the tuple's functions too (kernels.cu:11-13)
+    with pytest.raises(RuntimeError, match="must be a CUDA tensor"):
+        m.module_fp32[0](torch.zeros(1, 8, 4, 4), m.weight, m.theta)
+
+
+def test_state_dict_with_16_bit_theta_loads_as_fp32_values():
+    """A checkpoint whose theta was saved in a 16-bit type loads into the fp32 parameter: the
+    dtype stays fp32, the values are the rounded ones (the information is gone from the file)."""
+    C, K = 8, 15
+    angles = [math.pi * c / 8 for c in range(C)]
+    m = op.DepthwiseOrientedConv1d(C, C, K, groups=C, angle=angles)
+    sd = {k: v.clone() for k, v in m.state_dict().items()}
+    sd["theta"] = sd["theta"].to(torch.bfloat16)
+    m.load_state_dict(sd)
+    assert m.theta.dtype == torch.float32
+    assert torch.equal(m.theta.detach(), torch.tensor(angles).to(torch.bfloat16).float())

@@ -137,3 +137,71 @@ def test_training_step_and_stage_outputs():
             assert p.grad is None, name
         else:
             assert p.grad is not None and torch.isfinite(p.grad).all(), name
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("variant,autocast", [("1dpp", True), ("1dpp", False), ("1d", True)])
+def test_training_step_gradients_match_oracle(oracle, variant, autocast):
+    """One forward + backward + AdamW step of a reduced network, as the training configurations
+    run it (bf16 autocast over fp32 master weights, or plain fp32).  Every oriented convolution's
+    input, upstream gradient and the three gradients it produced are captured; each is checked
+    against the oracle's module_backward on the captured tensors (dwoconv1d.py:41-69)."""
+    from parity_util import assert_close, host
+
+    torch.manual_seed(3)
+    net = ConvNeXt1D(depths=(1, 2, 1, 1), dims=(16, 32, 64, 128), variant=variant, stem_dim1=16,
+                     num_classes=10, layer_scale_init_value=1.0).cuda().train()
+    for name, p in net.named_parameters():
+        if name.endswith("bias"):
+            torch.nn.init.normal_(p, std=0.1)
+    opt = torch.optim.AdamW(net.parameters(), lr=1e-3, weight_decay=0.05)
+    convs = [(n, m) for n, m in net.named_modules() if isinstance(m, DepthwiseOrientedConv1d)]
+    seen = {}
+
+    def capture_input(name):
+        # the convolution gets its own copy of the input, so the gradient seen on that copy is
+        # the convolution's dx alone (the block's residual branch reads the original)
+        def pre_hook(mod, inputs):
+            xi = inputs[0].clone()
+            rec = seen.setdefault(name, {})
+            rec["x"] = xi.detach().clone()
+            if xi.requires_grad:
+                xi.register_hook(lambda g: rec.__setitem__("dx", g.detach().clone()))
+            return (xi,)
+        return pre_hook
+
+    def capture_output(name):
+        def hook(mod, inputs, output):
+            rec = seen[name]
+            output.register_hook(lambda g: rec.__setitem__("dy", g.detach().clone()))
+        return hook
+
+    handles = [m.register_forward_pre_hook(capture_input(n)) for n, m in convs]
+    handles += [m.register_forward_hook(capture_output(n)) for n, m in convs]
+    imgs = torch.randn(4, 3, 64, 64, device="cuda")
+    labels = torch.randint(0, 10, (4,), device="cuda")
+    before = {n: m.weight.detach().clone() for n, m in convs}
+    opt.zero_grad(set_to_none=True)
+    with torch.autocast("cuda", dtype=torch.bfloat16, enabled=autocast):
+        loss = torch.nn.functional.cross_entropy(net(imgs).float(), labels)
+    loss.backward()
+    for h in handles:
+        h.remove()
+    assert len(seen) == len(convs) >= 7
+    for name, m in convs:
+        rec = seen[name]
+        dt = rec["x"].dtype
+        w, th = host(before[name]), host(m.theta)
+        dx, dw, db = oracle.module_backward(host(rec["dy"]), host(rec["x"]), w, th,
+                                            stride=m.stride[0], nhwc=m.nhwc,
+                                            resid=m.resid is not None)
+        tag = "%s %s %s" % (variant, name, dt)
+        assert m.weight.grad.dtype == torch.float32 and m.theta.grad is None
+        # dw/db: fp32 sums of products of the captured (already rounded) tensors
+        assert_close(host(m.weight.grad), dw, torch.float32, tag + " dw")
+        assert_close(host(m.bias.grad), db, torch.float32, tag + " db")
+        if "dx" in rec:
+            assert_close(host(rec["dx"]), dx, dt, tag + " dx")
+    opt.step()
+    for name, m in convs:
+        assert torch.isfinite(m.weight).all() and not torch.equal(m.weight.detach(), before[name])

@@ -98,6 +98,17 @@ def test_stage_shapes_k15(oracle, C, HW, nhwc, dtype):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
 @pytest.mark.parametrize("nhwc", [False, True], ids=["nchw", "nhwc"])
+@pytest.mark.parametrize("HW", [56, 28, 14])
+def test_reference_benchmark_shapes_k7(oracle, HW, nhwc, dtype):
+    """K = 7 at the extents of the reference's own micro-benchmark (analysis/benchmark.py:84-104):
+    the eight orientations, and the angles that script really passes (degrees read as radians)."""
+    _case(oracle, 3, 64, HW, HW, 7, 1, dtype, nhwc, canonical_theta(64), seed=HW + 7)
+    published = np.array([0, 22.5, 45, 66.75, 90, 112.5, 135, 157.5] * 2, dtype=np.float32)
+    _case(oracle, 2, 16, HW, HW, 7, 1, dtype, nhwc, published, seed=HW + 8)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("nhwc", [False, True], ids=["nchw", "nhwc"])
 @pytest.mark.parametrize("C,HW", [(48, 56), (64, 28), (96, 14), (128, 7)])
 def test_stage_shapes_reversed_orientations(oracle, C, HW, nhwc, dtype):
     """Angles of the layers turned by 90 degrees (models/convnext.py:159-160): half of them lie
@@ -232,70 +243,99 @@ def test_wgrad_is_deterministic():
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("nhwc", [False, True], ids=["nchw", "nhwc"])
 @pytest.mark.parametrize("C,HW", [(96, 56), (192, 28), (384, 14), (768, 7)])
-def test_full_size_properties(oracle, C, HW, dtype):
-    """Batch-64 stage shapes: size-independent properties on the full tensors
-    (adjoint identities, linearity in x) plus oracle parity on two whole images."""
+def test_full_size_all_ops_against_oracle(oracle, C, HW, nhwc, dtype):
+    """Batch-64 stage shapes, the tensors the roofline is measured on: every image of fprop and
+    dgrad (all image groups of every workgroup split, first and last batch included) and the
+    full-length wgrad / bias-gradient reduction against the double-accumulating oracle, plus
+    the size-independent properties (adjoint identities, exact linearity)."""
     N, K = 64, 31
     theta = canonical_theta(C)
-    g = torch.Generator(device="cuda").manual_seed(C)
-    x = torch.randn(N, C, HW, HW, device="cuda", generator=g).to(dtype)
-    dy = torch.randn(N, C, HW, HW, device="cuda", generator=g).to(dtype)
-    w = torch.randn(C, 1, 1, K, device="cuda", generator=g) * 0.02
+    rng = np.random.default_rng(C + HW)
+    x = rounded(rng.standard_normal((N, C, HW, HW)).astype(np.float32), dtype)
+    dy = rounded(rng.standard_normal((N, C, HW, HW)).astype(np.float32), dtype)
+    w = (rng.standard_normal((C, 1, 1, K)) * 0.02).astype(np.float32)
+    print("full size C%d %dx%d %s %s" % (C, HW, HW, dtype, "nhwc" if nhwc else "nchw"), flush=True)
+
+    def lay(a):
+        return np.ascontiguousarray(a.transpose(0, 2, 3, 1)) if nhwc else a
+
+    def unlay(t):
+        return t.permute(0, 3, 1, 2) if nhwc else t
+
     taps = op.build_taps(torch.from_numpy(theta), C, K).cuda()
-    y = op.fprop(x, w, taps)
-    dx = op.dgrad(dy, w, taps, (HW, HW))
-    dw, db = op.wgrad(dy, x, taps, K, with_bias=True)
+    xd, dyd, wd = dev(lay(x), dtype), dev(lay(dy), dtype), dev(w, torch.float32)
+    yd = op.fprop(xd, wd, taps, nhwc=nhwc)
+    dxd = op.dgrad(dyd, wd, taps, (HW, HW), nhwc=nhwc)
+    dwd, dbd = op.wgrad(dyd, xd, taps, K, nhwc=nhwc, with_bias=True)
     torch.cuda.synchronize()
+    nthr = min(16, oracle.max_threads())
+    assert_close(host(unlay(yd)), oracle.fprop(x, w, theta, threads=nthr), dtype, "fprop")
+    assert_close(host(unlay(dxd)), oracle.dgrad(dy, w, theta, threads=nthr), dtype, "dgrad")
+    # dw/db are fp32 sums of exact products of the (already rounded) inputs: fp32 tolerance
+    assert_close(host(dwd), oracle.wgrad(dy, x, theta, K, threads=nthr), torch.float32, "wgrad")
+    assert_close(host(dbd), oracle.bgrad(dy), torch.float32, "bgrad")
     # <y,dy> = <x,dx> = <w,dw>; terms are O(1) random so compare against sqrt(#terms) scale
-    a = (y.double() * dy.double()).sum().item()
-    b = (x.double() * dx.double()).sum().item()
-    c = (w.double() * dw.double()).sum().item()
-    scale = math.sqrt((y.double() ** 2).sum().item() * (dy.double() ** 2).sum().item())
+    a = (yd.double() * dyd.double()).sum().item()
+    b = (xd.double() * dxd.double()).sum().item()
+    c = (wd.double() * dwd.double()).sum().item()
+    scale = math.sqrt((yd.double() ** 2).sum().item() * (dyd.double() ** 2).sum().item())
     tol = TOL[dtype]
     assert abs(a - c) <= tol * scale and abs(a - b) <= tol * scale, (a, b, c, scale)
-    assert_close(host(db), host(dy.double().sum((0, 2, 3))), torch.float32, "db")
     # linearity: fprop(2x) = 2 fprop(x) exactly (power-of-two scaling commutes with rounding)
-    assert torch.equal(op.fprop(x * 2, w, taps), y * 2)
-    # two whole images against the oracle
-    xs, dys = host(x[5:7]), host(dy[5:7])
-    assert_close(host(y[5:7]), oracle.fprop(xs, host(w), theta, threads=8), dtype, "fprop n=5,6")
-    assert_close(host(dx[5:7]), oracle.dgrad(dys, host(w), theta, threads=8), dtype, "dgrad n=5,6")
+    assert torch.equal(op.fprop(xd * 2, wd, taps, nhwc=nhwc), yd * 2)
 
 
-def test_full_size_wgrad_against_oracle(oracle):
-    """wgrad at the full batch-64 reduction length for the two smallest stage shapes
-    (the oracle needs the whole batch; these finish in seconds on the host)."""
-    for C, HW in [(768, 7), (384, 14)]:
-        theta = canonical_theta(C)
-        rng = np.random.default_rng(C)
-        x = rng.standard_normal((64, C, HW, HW)).astype(np.float32)
-        dy = rng.standard_normal((64, C, HW, HW)).astype(np.float32)
-        taps = op.build_taps(torch.from_numpy(theta), C, 31).cuda()
-        dw, _ = op.wgrad(dev(dy, torch.float32), dev(x, torch.float32), taps, 31)
-        assert_close(host(dw), oracle.wgrad(dy, x, theta, 31, threads=8), torch.float32,
-                     "wgrad C%d %d^2" % (C, HW))
+# The operator launches of the two training configurations, at reduced batch, bf16 (what the
+# networks run under autocast / after .to(bfloat16)): ConvNeXt-B-1D++ at 224 x 224 -- second
+# convolutions NHWC K=31 with a residual tap on the 4x-expanded channels, first convolutions
+# NCHW K=15, the K=15 stem -- and ConvNeXt-T-1D at 512 x 512 -- stages of 128, 64, 32, 16
+# squared and the K=31 stem.  Angles are the networks' contiguous groups, odd layers turned by
+# 90 degrees (models/convnext.py:60-77).
+_TRAINING_LAUNCHES = [
+    # N, C, HW, K, stride, nhwc
+    (2, 512, 56, 31, 1, True), (2, 1024, 28, 31, 1, True), (2, 2048, 14, 31, 1, True),
+    (3, 4096, 7, 31, 1, True),
+    (2, 128, 56, 15, 1, False), (2, 256, 28, 15, 1, False), (2, 512, 14, 15, 1, False),
+    (3, 1024, 7, 15, 1, False),
+    (2, 64, 224, 15, 2, True), (2, 64, 112, 15, 2, True),
+    (2, 96, 128, 31, 1, False), (2, 192, 64, 31, 1, False), (2, 384, 32, 31, 1, False),
+    (3, 768, 16, 31, 1, False),
+    (1, 64, 512, 31, 2, True), (2, 64, 256, 31, 2, True), (2, 64, 224, 31, 2, True),
+]
+
+
+@pytest.mark.parametrize("offset", [0.0, 0.5], ids=["even", "odd"])
+@pytest.mark.parametrize("N,C,HW,K,stride,nhwc", _TRAINING_LAUNCHES,
+                         ids=["%dx%d_k%d_s%d_%s" % (c, hw, k, s, "nhwc" if l else "nchw")
+                              for _, c, hw, k, s, l in _TRAINING_LAUNCHES])
+def test_training_configuration_launch_shapes(oracle, N, C, HW, K, stride, nhwc, offset):
+    if offset == 0.5 and HW > 128:
+        pytest.skip("the two stem layers differ by the same 90 degrees; one is enough at this size")
+    _case(oracle, N, C, HW, HW, K, stride, torch.bfloat16, nhwc, grouped_theta(C, offset),
+          seed=C + HW + K, threads=min(16, oracle.max_threads()))
 
 
 @pytest.mark.gpu
 def test_step_captured_in_a_graph_replays_identically():
-    """fprop + dgrad + wgrad through the C ABI captured into one graph (the library launches
-    only kernels, nothing a capture refuses): three replays, each after unrelated eager work and
+    """fprop + dgrad + wgrad through the C ABI captured into one graph.  The first thing the
+    capture contains is the first call of each entry point in this process for this shape: the
+    per-device set-up (occupancy queries, kernel attributes) was done by dwo_init, so the calls
+    only launch kernels.  Three replays, each after unrelated eager work and
     a synchronisation, on fresh inputs written into the captured buffers, must equal the eager
     results bit for bit."""
     torch.manual_seed(5)
-    N, C, HW, K = 4, 96, 28, 31
+    N, C, HW, K = 4, 80, 28, 15  # a (K, extent) no other test of this module launches first
     theta = torch.from_numpy(canonical_theta(C))
     taps = op.build_taps(theta, C, K).cuda()
     w = (torch.randn(C, 1, 1, K, device="cuda") * 0.02)
     x = torch.randn(N, C, HW, HW, device="cuda")
     dy = torch.randn(N, C, HW, HW, device="cuda")
     stream = torch.cuda.Stream()
+    from oriented1d_amd import _lib
+    _lib.ready(x.device)
     with torch.cuda.stream(stream):
-        for _ in range(2):  # first calls query occupancy and set kernel attributes: not capturable
-            op.fprop(x, w, taps, 1)
-            op.dgrad(dy, w, taps, (HW, HW), 1)
-            op.wgrad(dy, x, taps, K, 1, with_bias=True)
         torch.cuda.synchronize()
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph, stream=stream):

@@ -109,7 +109,8 @@ def test_theta90_is_flipped_vertical_conv2d(oracle, stride):
     np.testing.assert_allclose(got, ref, rtol=0, atol=1e-12)
 
 
-@pytest.mark.parametrize("stride,HW", [(1, (10, 12)), (1, (7, 7)), (2, (12, 8)), (2, (9, 11))])
+@pytest.mark.parametrize("stride,HW", [(1, (10, 12)), (1, (7, 7)), (2, (12, 8)), (2, (9, 11)),
+                                       (4, (16, 12)), (4, (13, 18))])
 def test_any_theta_matches_dense_2d_kernel_and_its_autograd(oracle, stride, HW):
     """fprop == conv2d with the taps scattered into a dense 2-D kernel; autograd of that
     library op pins dgrad and wgrad (incl. duplicate taps and the ceil(H/stride) extent)."""
@@ -151,7 +152,7 @@ def test_impulse_response(oracle):
     np.testing.assert_allclose(y[0], exp, rtol=0, atol=1e-12)
 
 
-@pytest.mark.parametrize("stride", [1, 2])
+@pytest.mark.parametrize("stride", [1, 2, 4])
 def test_adjoint_identities(oracle, stride):
     """<fprop(x),dy> = <x,dgrad(dy)> = <w,wgrad(dy,x)>."""
     rng = np.random.default_rng(3)
@@ -161,7 +162,7 @@ def test_adjoint_identities(oracle, stride):
     y = oracle.fprop(x, w, theta, stride)
     dy = _rand(y.shape, 22)
     a = (y * dy).sum()
-    b = (x.astype(np.float64) * oracle.dgrad(dy, w, theta, stride)).sum()
+    b = (x.astype(np.float64) * oracle.dgrad(dy, w, theta, stride, in_hw=(H, W))).sum()
     c = (w.astype(np.float64) * oracle.wgrad(dy, x, theta, S, stride).reshape(C, S)).sum()
     assert abs(a - b) < 1e-9 * max(1, abs(a)) and abs(a - c) < 1e-9 * max(1, abs(a))
 
@@ -174,7 +175,7 @@ def test_stride_subsamples_stride1(oracle):
         np.testing.assert_array_equal(oracle.fprop(x, w, theta, stride), y1[..., ::stride, ::stride])
 
 
-@pytest.mark.parametrize("stride,HW", [(1, (6, 7)), (2, (6, 8)), (2, (5, 7))])
+@pytest.mark.parametrize("stride,HW", [(1, (6, 7)), (2, (6, 8)), (2, (5, 7)), (4, (8, 8)), (4, (9, 6))])
 def test_c_oracle_equals_python_brute_force(oracle, stride, HW):
     rng = np.random.default_rng(9)
     theta = np.concatenate([np.array(PI8[1:4]), rng.uniform(0, math.pi, 2).astype(np.float32)])
