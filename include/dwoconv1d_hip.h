@@ -59,6 +59,7 @@ extern "C" {
 #define DWO_ERR_BAD_LAYOUT (-6)
 #define DWO_ERR_SCRATCH_TOO_SMALL (-7)
 #define DWO_ERR_BAD_TAPS (-8)     /* host-side tap blob does not match C,K */
+#define DWO_ERR_STATIC_SCRATCH_LIMIT (-9) /* dwo_wgrad_static: partial sums exceed the static scratch */
 
 #define DWO_MAX_K 63
 
@@ -130,6 +131,22 @@ int dwo_wgrad(const void *dy, const void *x, const void *taps, float *dw, float 
               void *scratch, size_t scratch_bytes,
               int N, int C, int H, int W, int K, int stride, int dtype, int layout,
               void *stream);
+
+/*
+ * wgrad without any device allocation by caller or library -- no counterpart in the reference.
+ * It is for callers that cannot allocate: code under stream capture, tight serving loops,
+ * harnesses that forbid hipMalloc.  Same results as dwo_wgrad (bit for bit: the same kernels),
+ * with the partial sums kept in a DWO_STATIC_SCRATCH_BYTES array in device memory that is part
+ * of the library image (one copy per GPU, held until the process ends).  Shapes whose
+ * dwo_wgrad_scratch_bytes exceed it are refused with DWO_ERR_STATIC_SCRATCH_LIMIT.  Every call on a
+ * GPU shares that GPU's array: calls that overlap in time on one GPU (different streams or
+ * threads) race; calls on one stream are ordered.  Nothing in the array has to survive between
+ * calls and nothing in it has to be cleared.
+ */
+#define DWO_STATIC_SCRATCH_BYTES (8u << 20)
+int dwo_wgrad_static(const void *dy, const void *x, const void *taps, float *dw, float *db,
+                     int N, int C, int H, int W, int K, int stride, int dtype, int layout,
+                     void *stream);
 
 /*
  * fprop of a pointwise-projected NHWC tensor without materialising it: y = fprop(pw(x)) with

@@ -23,6 +23,7 @@ SIGNATURES = {
     "dwo_dgrad": (_i, [_vp, _vp, _vp, _vp] + [_i] * 8 + [_vp]),
     "dwo_wgrad_scratch_bytes": (_sz, [_i] * 8),
     "dwo_wgrad": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _sz] + [_i] * 8 + [_vp]),
+    "dwo_wgrad_static": (_i, [_vp, _vp, _vp, _vp, _vp] + [_i] * 8 + [_vp]),
     "dwo_pointwise_fprop_nhwc": (_i, [_vp] * 7 + [_i] * 8 + [_vp]),
     "dwo_layernorm_nhwc": (_i, [_vp, _vp, _vp, _vp, _sz, _i, ctypes.c_float, _i, _i, _vp]),
     "dwo_nchw_layernorm_nhwc": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, ctypes.c_float, _i, _vp]),

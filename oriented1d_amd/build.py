@@ -49,9 +49,11 @@ def _run(cmd, verbose):
         print(err)
 
 
-def build(verbose=False, jobs=None):
+def build(verbose=False, jobs=None, only=None):
     """Compile csrc/dwo_api.hip and one csrc/dwo_inst.hip object per (element type, plane
-    extent) in parallel, then link libdwoconv1d_hip.so into the package directory."""
+    extent) in parallel, then link libdwoconv1d_hip.so into the package directory.  ``only``
+    (substrings of object names, e.g. ``["dwo_api", "float_k31_56"]``) recompiles just those
+    units and links them with the objects a previous full build left in place."""
     from concurrent.futures import ThreadPoolExecutor
 
     objdir = os.path.join(HERE, "build")
@@ -65,9 +67,15 @@ def build(verbose=False, jobs=None):
                           os.path.join(objdir, "dwo_inst_%s_k%d_%dx%d.o" % (t, K, H, W)),
                           ["-DDWO_INST_T=" + t, "-DDWO_INST_K=%d" % K, "-DDWO_INST_H=%d" % H,
                            "-DDWO_INST_W=%d" % W]))
-    jobs = jobs or min(len(units), max(1, min(16, os.cpu_count() or 1)))
+    todo = units
+    if only:
+        todo = [u for u in units if any(tag in os.path.basename(u[1]) for tag in only)]
+        missing = [u[1] for u in units if u not in todo and not os.path.exists(u[1])]
+        if missing:
+            raise RuntimeError("a partial build needs the objects of a full one; missing " + missing[0])
+    jobs = jobs or min(len(todo), max(1, min(16, os.cpu_count() or 1)))
     with ThreadPoolExecutor(jobs) as pool:
-        list(pool.map(lambda u: _run(common + u[2] + [u[0], "-o", u[1]], verbose), units))
+        list(pool.map(lambda u: _run(common + u[2] + [u[0], "-o", u[1]], verbose), todo))
     _run([hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC"] + [u[1] for u in units] +
          ["-o", LIB + ".tmp"], verbose)
     os.replace(LIB + ".tmp", LIB)
@@ -75,4 +83,6 @@ def build(verbose=False, jobs=None):
 
 
 if __name__ == "__main__":
-    print(build(verbose=True))
+    import sys
+
+    print(build(verbose="-q" not in sys.argv[1:], only=[a for a in sys.argv[1:] if a != "-q"] or None))

@@ -331,6 +331,28 @@ int wgrad_dispatch(const void *dy, const void *x, const void *taps, float *dw, f
     }
 }
 
+// Partial sums of dwo_wgrad_static.  One copy per GPU, held until the process ends.  The name
+// is only a host-side handle: the memory's address on the current device comes from
+// hipGetSymbolAddress (static_scratch below) and that pointer is what the kernels are given.
+static __device__ __align__(256) unsigned char g_wgrad_scratch[DWO_STATIC_SCRATCH_BYTES];
+void *g_wgrad_scratch_ptr[kMaxDevices];
+
+int static_scratch(void **out) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    if (dev < 0 || dev >= kMaxDevices) return DWO_ERR_BAD_SHAPE;
+    void *p = __atomic_load_n(&g_wgrad_scratch_ptr[dev], __ATOMIC_ACQUIRE);
+    if (p == nullptr) {
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(g_wgrad_scratch));
+        if (e != hipSuccess) return (int)e;
+        if (p == nullptr) return (int)hipErrorInvalidSymbol;
+        __atomic_store_n(&g_wgrad_scratch_ptr[dev], p, __ATOMIC_RELEASE);
+    }
+    *out = p;
+    return DWO_OK;
+}
+
 // One-time set-up of every kernel on the current device (see per_device_once): the launchers
 // are called with an empty batch, which stops them after their set-up.
 template <typename T>
@@ -367,6 +389,9 @@ extern "C" {
 
 int dwo_init(void) {
     begin_call();
+    void *scratch = nullptr;  // the static wgrad scratch's address on this device
+    const int rc = static_scratch(&scratch);
+    if (rc != DWO_OK) return rc;
     // (the set-up calls leave their own failures in the runtime's last-error slot)
     (void)init_type<float>();
     (void)init_type<bf16_t>();
@@ -387,6 +412,8 @@ const char *dwo_status_string(int status) {
         case DWO_ERR_BAD_LAYOUT: return "unsupported layout";
         case DWO_ERR_SCRATCH_TOO_SMALL: return "wgrad scratch buffer too small";
         case DWO_ERR_BAD_TAPS: return "tap table does not match C and K";
+        case DWO_ERR_STATIC_SCRATCH_LIMIT:
+            return "wgrad partial sums exceed the static scratch (DWO_STATIC_SCRATCH_BYTES)";
         default: break;
     }
     if (status > 0) return hipGetErrorString((hipError_t)status);
@@ -511,6 +538,20 @@ int dwo_wgrad(const void *dy, const void *x, const void *taps, float *dw, float 
     if (!dy || !x || !taps || !dw || !scratch) return DWO_ERR_NULL_POINTER;
     if (scratch_bytes < dwo_wgrad_scratch_bytes(N, C, H, W, K, stride, dtype, layout))
         return DWO_ERR_SCRATCH_TOO_SMALL;
+    return wgrad_dispatch(dy, x, taps, dw, db, scratch, N, C, H, W, K, stride, dtype, layout,
+                          (hipStream_t)stream);
+}
+
+int dwo_wgrad_static(const void *dy, const void *x, const void *taps, float *dw, float *db, int N,
+                     int C, int H, int W, int K, int stride, int dtype, int layout, void *stream) {
+    int rc = check_common(N, C, H, W, K, stride, dtype, layout);
+    if (rc != DWO_OK) return rc;
+    if (!dy || !x || !taps || !dw) return DWO_ERR_NULL_POINTER;
+    if (dwo_wgrad_scratch_bytes(N, C, H, W, K, stride, dtype, layout) > DWO_STATIC_SCRATCH_BYTES)
+        return DWO_ERR_STATIC_SCRATCH_LIMIT;
+    void *scratch = nullptr;
+    rc = static_scratch(&scratch);
+    if (rc != DWO_OK) return rc;
     return wgrad_dispatch(dy, x, taps, dw, db, scratch, N, C, H, W, K, stride, dtype, layout,
                           (hipStream_t)stream);
 }
