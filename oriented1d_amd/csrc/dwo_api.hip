@@ -6,6 +6,8 @@
 #include <stdlib.h>
 #include <string.h>
 
+#include <atomic>
+
 #include "dwo_common.h"
 #include "dwo_generic.h"
 #include "dwo_nhwc.h"
@@ -92,10 +94,11 @@ int try_plane_conv(int op, const void *src, const float *w, const float *bias, c
 
 template <typename T>
 int try_plane_wgrad(const void *x, const void *dy, const void *taps, float *part, float *dw,
-                    float *db, int *groups, const ConvDims &d, hipStream_t st) {
+                    float *db, unsigned *tickets, int *groups, const ConvDims &d, hipStream_t st) {
 #define DWO_MATCH(K_, H_, W_)                                                               \
     if (d.K == K_ && d.H == H_ && d.W == W_)                                                \
-        return launch_plane_wgrad<T, K_, H_, W_>(x, dy, taps, part, dw, db, d.N, d.C, groups, st);
+        return launch_plane_wgrad<T, K_, H_, W_>(x, dy, taps, part, dw, db, tickets, d.N, d.C, \
+                                                 groups, st);
     DWO_PLANE_SHAPES(DWO_MATCH)
 #undef DWO_MATCH
     return -100;
@@ -138,11 +141,12 @@ int nhwc_plane_batch(const ConvDims &d, int layout) {
 
 template <typename T>
 int try_nhwc_plane_wgrad(const void *x, const void *dy, const void *taps, float *part, float *dw,
-                         float *db, int *groups, const ConvDims &d, hipStream_t st) {
+                         float *db, unsigned *tickets, int *groups, const ConvDims &d,
+                         hipStream_t st) {
 #define DWO_MATCH(K_, H_, W_)                                                                    \
     if (d.K == K_ && d.H == H_ && d.W == W_)                                                     \
-        return launch_nhwc_plane_wgrad<T, K_, H_, W_>(x, dy, taps, part, dw, db, d.N, d.C, groups, \
-                                                      st);
+        return launch_nhwc_plane_wgrad<T, K_, H_, W_>(x, dy, taps, part, dw, db, tickets, d.N, d.C, \
+                                                      groups, st);
     DWO_PLANE_SHAPES(DWO_MATCH)
 #undef DWO_MATCH
     return -100;
@@ -271,18 +275,49 @@ int dgrad_t(const void *dy, const float *w, const void *taps, void *dx, const Co
     return launch_status();
 }
 
+// Ticket counters of the plane wgrad kernels (wgrad_finish): one counter per channel block and
+// launch.  They live in the library's device image, zero when the library is loaded, and every
+// launch leaves its counters at zero again.  Launches that may run at the same time must not
+// share counters, so each call takes the next of kTicketSlots rows; a row is reused
+// kTicketSlots calls later, long after the launch that used it has drained (a device runs a
+// handful of kernels at once).  Shapes with more channel blocks than a row holds, and devices
+// where the symbol cannot be resolved, take the separate reduction kernel instead.
+constexpr int kTicketSlots = 64, kTicketRow = 4096;
+static __device__ unsigned g_tickets[kTicketSlots * kTicketRow];
+unsigned *g_tickets_ptr[kMaxDevices];
+std::atomic<unsigned> g_ticket_next{0};
+
+unsigned *ticket_row(int blocks) {
+    if (blocks > kTicketRow) return nullptr;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return nullptr;
+    unsigned *p = __atomic_load_n(&g_tickets_ptr[dev], __ATOMIC_ACQUIRE);
+    if (p == nullptr) {
+        void *sym = nullptr;
+        if (hipGetSymbolAddress(&sym, HIP_SYMBOL(g_tickets)) != hipSuccess || sym == nullptr) {
+            (void)hipGetLastError();
+            return nullptr;
+        }
+        p = (unsigned *)sym;
+        __atomic_store_n(&g_tickets_ptr[dev], p, __ATOMIC_RELEASE);
+    }
+    return p + (size_t)(g_ticket_next.fetch_add(1, std::memory_order_relaxed) % kTicketSlots) * kTicketRow;
+}
+
 template <typename T>
 int wgrad_t(const void *dy, const void *x, const void *taps, float *dw, float *db, void *scratch,
             const ConvDims &d, int layout, hipStream_t st) {
     float *part = (float *)scratch;
     int rc, NG = 0;
-    bool direct = false;  // a single group per channel: stage 1 wrote dw / db itself
+    bool direct = false;  // stage 1 wrote dw / db itself (one group per channel, or tickets)
     if (plane_batch(d, layout) != 0) {
-        rc = try_plane_wgrad<T>(x, dy, taps, part, dw, db, &NG, d, st);
-        direct = NG == 1;
+        unsigned *tickets = ticket_row(d.C);
+        rc = try_plane_wgrad<T>(x, dy, taps, part, dw, db, tickets, &NG, d, st);
+        direct = NG == 1 || tickets != nullptr;
     } else if (nhwc_plane_batch(d, layout) != 0) {
-        rc = try_nhwc_plane_wgrad<T>(x, dy, taps, part, dw, db, &NG, d, st);
-        direct = NG == 1;
+        unsigned *tickets = ticket_row(d.C / kSliceCh);
+        rc = try_nhwc_plane_wgrad<T>(x, dy, taps, part, dw, db, tickets, &NG, d, st);
+        direct = NG == 1 || tickets != nullptr;
     } else if (tile_covers(d, layout, sizeof(T))) {
         rc = launch_tile_wgrad<T>(x, dy, taps, part, &NG, d, layout == DWO_NCHW, st);
     } else if (layout == DWO_NHWC && nhwc_has_k(d.K)) {
@@ -362,11 +397,11 @@ int init_type() {
     rc |= launch_plane_conv<T, K_, H_, W_>(OP_FPROP, nullptr, nullptr, nullptr, nullptr, nullptr, \
                                            0, 1, nullptr);                                        \
     rc |= launch_plane_wgrad<T, K_, H_, W_>(nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, \
-                                            0, 1, &ng, nullptr);                                  \
+                                            nullptr, 0, 1, &ng, nullptr);                         \
     rc |= launch_nhwc_plane_conv<T, K_, H_, W_>(OP_FPROP, nullptr, nullptr, nullptr, nullptr,     \
                                                 nullptr, 0, kSliceCh, nullptr);                   \
     rc |= launch_nhwc_plane_wgrad<T, K_, H_, W_>(nullptr, nullptr, nullptr, nullptr, nullptr,     \
-                                                 nullptr, 0, kSliceCh, &ng, nullptr);
+                                                 nullptr, nullptr, 0, kSliceCh, &ng, nullptr);
     DWO_PLANE_SHAPES(DWO_PREP)
 #undef DWO_PREP
     ConvDims d = make_dims(1, kSliceCh, 8, 8, 7, 2);
@@ -392,6 +427,7 @@ int dwo_init(void) {
     void *scratch = nullptr;  // the static wgrad scratch's address on this device
     const int rc = static_scratch(&scratch);
     if (rc != DWO_OK) return rc;
+    (void)ticket_row(1);  // and the ticket counters' (a row taken here is simply skipped)
     // (the set-up calls leave their own failures in the runtime's last-error slot)
     (void)init_type<float>();
     (void)init_type<bf16_t>();
@@ -422,7 +458,7 @@ const char *dwo_status_string(int status) {
 
 size_t dwo_taps_bytes(int C, int K) {
     if (C < 1 || K < 1 || K > DWO_MAX_K || (K & 1) == 0) return 0;
-    return kTapsHeaderBytes + taps_dhdw_bytes(C, K) + 2 * taps_class_bytes(C) + taps_extent_bytes(C);
+    return kTapsHeaderBytes + taps_dhdw_bytes(C, K) + 3 * taps_class_bytes(C) + taps_extent_bytes(C);
 }
 
 int dwo_build_taps(const float *theta_host, int C, int K, void *taps_host) {
@@ -470,6 +506,13 @@ int dwo_build_taps(const float *theta_host, int C, int K, void *taps_host) {
             next[k] = c + 1;
             if (c < C) order[placed++] = c;
         }
+    }
+    // and the channels sorted by class: 0, .., 7, then the non-canonical ones (stable)
+    int32_t *sorted = const_cast<int32_t *>(taps_sorted(taps_host, C, K));
+    for (int k = 0, placed = 0; k < 9; k++) {
+        const int want = k < 8 ? k : -1;
+        for (int c = 0; c < C; c++)
+            if (cls[c] == want) sorted[placed++] = c;
     }
     hdr[7] = hdr[6] + (int32_t)taps_class_bytes(C);
     int8_t *extent = (int8_t *)taps_host + hdr[7];

@@ -16,14 +16,19 @@ namespace dwo {
 //                              (k * 22.5 degrees), or -1 when the pattern is not canonical;
 //                              padded to 16 bytes
 //   int32 order[C]             the channels in an order that cycles through the orientation
-//                              classes (class 0, 1, .., 7, other, 0, 1, ..): per-channel
-//                              workgroups take their channel from it, so that whatever way the
-//                              angles are laid out over the channels, neighbouring workgroup
-//                              ids (hence every XCD and CU) get a mix of orientations
+//                              classes (class 0, 1, .., 7, other, 0, 1, ..): the per-channel
+//                              workgroups of fprop and dgrad take their channel from it, so that
+//                              whatever way the angles are laid out over the channels,
+//                              neighbouring workgroup ids (hence every XCD and CU) get a mix of
+//                              orientations
 //   int8  extent[C][2]         (max |dh|, max |dw|) over the channel's taps, padded to 16 bytes
+//   int32 sorted[C]            the channels sorted by orientation class (class 0, .., 7, then the
+//                              non-canonical ones): the per-channel workgroups of wgrad take
+//                              their channel from it, so that the workgroups sharing a CU run
+//                              the same class; padded to 16 bytes
 // ---------------------------------------------------------------------------------------------
 constexpr int32_t kTapsMagic = 0x44574f31;  // "DWO1"
-constexpr int32_t kTapsVersion = 4;
+constexpr int32_t kTapsVersion = 5;
 constexpr int kTapsHeaderInts = 8;
 constexpr int kTapsHeaderBytes = kTapsHeaderInts * 4;
 
@@ -46,6 +51,11 @@ __host__ __device__ inline size_t taps_extent_bytes(int C) {
 __host__ __device__ inline const int8_t *taps_extent(const void *blob, int C, int K) {
     return reinterpret_cast<const int8_t *>(blob) + kTapsHeaderBytes + taps_dhdw_bytes(C, K) +
            2 * taps_class_bytes(C);
+}
+__host__ __device__ inline const int32_t *taps_sorted(const void *blob, int C, int K) {
+    return reinterpret_cast<const int32_t *>(reinterpret_cast<const int8_t *>(blob) +
+                                             kTapsHeaderBytes + taps_dhdw_bytes(C, K) +
+                                             2 * taps_class_bytes(C) + taps_extent_bytes(C));
 }
 __host__ __device__ inline const int32_t *taps_order(const void *blob, int C, int K) {
     return reinterpret_cast<const int32_t *>(reinterpret_cast<const int8_t *>(blob) +

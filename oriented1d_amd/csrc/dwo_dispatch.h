@@ -44,7 +44,7 @@ int launch_plane_conv(int op, const void *src, const float *w, const float *bias
                       void *dst, int N, int C, hipStream_t st);
 template <typename T, int K, int H, int W>
 int launch_plane_wgrad(const void *x, const void *dy, const void *taps, float *part, float *dw,
-                       float *db, int N, int C, int *groups_out, hipStream_t st);
+                       float *db, unsigned *tickets, int N, int C, int *groups_out, hipStream_t st);
 
 // NHWC, C a multiple of 4: channel-slice workgroups over the same LDS planes
 template <typename T, int K, int H, int W>
@@ -53,21 +53,23 @@ int launch_nhwc_plane_conv(int op, const void *src, const float *w, const float 
 
 template <typename T, int K, int H, int W>
 int launch_nhwc_plane_wgrad(const void *x, const void *dy, const void *taps, float *part, float *dw,
-                            float *db, int N, int C, int *groups_out, hipStream_t st);
+                            float *db, unsigned *tickets, int N, int C, int *groups_out,
+                            hipStream_t st);
 
 #define DWO_DECLARE(T, K, H, W)                                                                   \
     extern template int launch_plane_conv<T, K, H, W>(int, const void *, const float *,           \
                                                       const float *, const void *, void *, int,   \
                                                       int, hipStream_t);                          \
     extern template int launch_plane_wgrad<T, K, H, W>(const void *, const void *, const void *,  \
-                                                       float *, float *, float *, int, int,       \
-                                                       int *, hipStream_t);                       \
+                                                       float *, float *, float *, unsigned *,     \
+                                                       int, int, int *, hipStream_t);             \
     extern template int launch_nhwc_plane_conv<T, K, H, W>(int, const void *, const float *,      \
                                                            const float *, const void *, void *,   \
                                                            int, int, hipStream_t);        \
     extern template int launch_nhwc_plane_wgrad<T, K, H, W>(const void *, const void *,           \
                                                             const void *, float *, float *,       \
-                                                            float *, int, int, int *, hipStream_t);
+                                                            float *, unsigned *, int, int, int *, \
+                                                            hipStream_t);
 #define DWO_DECLARE_ALL(K, H, W) \
     DWO_DECLARE(float, K, H, W) DWO_DECLARE(bf16_t, K, H, W) DWO_DECLARE(f16_t, K, H, W)
 DWO_PLANE_SHAPES(DWO_DECLARE_ALL)

@@ -7,11 +7,11 @@ namespace dwo {
 template int launch_plane_conv<DWO_INST_T, DWO_INST_K, DWO_INST_H, DWO_INST_W>(
     int, const void *, const float *, const float *, const void *, void *, int, int, hipStream_t);
 template int launch_plane_wgrad<DWO_INST_T, DWO_INST_K, DWO_INST_H, DWO_INST_W>(
-    const void *, const void *, const void *, float *, float *, float *, int, int, int *,
+    const void *, const void *, const void *, float *, float *, float *, unsigned *, int, int, int *,
     hipStream_t);
 template int launch_nhwc_plane_conv<DWO_INST_T, DWO_INST_K, DWO_INST_H, DWO_INST_W>(
     int, const void *, const float *, const float *, const void *, void *, int, int, hipStream_t);
 template int launch_nhwc_plane_wgrad<DWO_INST_T, DWO_INST_K, DWO_INST_H, DWO_INST_W>(
-    const void *, const void *, const void *, float *, float *, float *, int, int, int *,
+    const void *, const void *, const void *, float *, float *, float *, unsigned *, int, int, int *,
     hipStream_t);
 }  // namespace dwo

@@ -308,7 +308,7 @@ int launch_nhwc_plane_conv(int op, const void *src, const float *w, const float 
     const int slots = per_device_once(cache, [&] {
         allow_large_lds(nhwc_plane_kernel<OP_FPROP, T, K, H, W>, lds);
         allow_large_lds(nhwc_plane_kernel<OP_DGRAD, T, K, H, W>, lds);
-        return resident_slots(nhwc_plane_kernel<OP_FPROP, T, K, H, W>, NT, lds);
+        return resident_slots(nhwc_plane_kernel<OP_FPROP, T, K, H, W>, NT, lds) & 0xffff;
     });
     if (N == 0) return 0;  // set-up only
     const int nslices = C / kSliceCh;
@@ -440,6 +440,7 @@ __device__ __forceinline__ void wgrad_epilogue_sub(float (&acc)[K + 1], float *l
             for (int w = 0; w < NWS; w++) t += lds[(sub * NWS + w) * (K + 1) + slot];
         out.put(c, (int)stid, group, K, t);
     }
+    wgrad_finish<K>(out, lds, (c - sub) / kSliceCh, c - sub, kSliceCh);
 }
 
 // Barriers per batch are the same in every body: two per phase.
@@ -640,20 +641,21 @@ __global__ __launch_bounds__((NhwcTile<H, W>::NT)) void nhwc_plane_wgrad_kernel(
 // Same contract as launch_plane_wgrad.
 template <typename T, int K, int H, int W>
 int launch_nhwc_plane_wgrad(const void *x, const void *dy, const void *taps, float *part, float *dw,
-                            float *db, int N, int C, int *groups_out, hipStream_t st) {
+                            float *db, unsigned *tickets, int N, int C, int *groups_out,
+                            hipStream_t st) {
     constexpr int NT = NhwcTile<H, W>::NT, PBI = NhwcTile<H, W>::PBI;
     const size_t lds = nhwc_plane_wgrad_lds_bytes<K, H, W>();
     static int cache[kMaxDevices];
     const int slots = per_device_once(cache, [&] {
         allow_large_lds(nhwc_plane_wgrad_kernel<T, K, H, W>, lds);
-        return resident_slots(nhwc_plane_wgrad_kernel<T, K, H, W>, NT, lds);
+        return resident_slots(nhwc_plane_wgrad_kernel<T, K, H, W>, NT, lds) & 0xffff;
     });
     if (N == 0) return 0;  // set-up only
     const int nslices = C / kSliceCh;
     const int groups = plane_groups(N, nslices, PBI, slots);
     *groups_out = groups;
     nhwc_plane_wgrad_kernel<T, K, H, W><<<dim3(nslices * groups), dim3(NT), lds, st>>>(
-        (const T *)x, (const T *)dy, taps, WgradOut{part, dw, db, groups}, N, C);
+        (const T *)x, (const T *)dy, taps, WgradOut{part, dw, db, groups, tickets}, N, C);
     const hipError_t e = hipGetLastError();
     return e == hipSuccess ? 0 : (int)e;
 }

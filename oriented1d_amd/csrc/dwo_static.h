@@ -11,7 +11,13 @@
 // Register budget of the plane kernels: at least six waves per SIMD, i.e. three 448-thread
 // workgroups per CU (seven would need 72 registers and spill).
 #define DWO_WPE 6
+#ifndef DWO_WPE_WGRAD
 #define DWO_WPE_WGRAD 6
+#endif
+// batches in flight from HBM per tensor in the wgrad kernels (register sets per tensor)
+#ifndef DWO_WGRAD_DEPTH
+#define DWO_WGRAD_DEPTH 1
+#endif
 
 #include "dwo_common.h"
 #include "dwo_dispatch.h"
@@ -122,9 +128,10 @@ constexpr int max_plane_floats(std::integer_sequence<int, Os...>) {
     ((m = cmax(m, orient_class(Os) == CLS_H ? Geo<Os, K, tile_L<H, W>(Os), H, W, true>::PLANE : 0)), ...);
     return m;
 }
+// (a multiple of four words: planes keep the 16-byte alignment that wide LDS writes need)
 template <int K, int H, int W>
 constexpr int plane_floats() {
-    return max_plane_floats<K, H, W>(std::make_integer_sequence<int, 8>{});
+    return (max_plane_floats<K, H, W>(std::make_integer_sequence<int, 8>{}) + 3) & ~3;
 }
 
 // scalar stores of single results (4-byte ones non-temporal, like the vector stores)
@@ -195,8 +202,17 @@ struct Stager {
                 if constexpr (W % VL == 0) {
                     const unsigned r = g / (W / VL), w0 = (g % (W / VL)) * VL;
                     float *q = plane + Map::index(r, w0);
+                    if constexpr (VL == 4 && Map::kWide && PLS % 4 == 0) {
+                        // the chunk's four words are adjacent and 16-byte aligned in LDS: one
+                        // wide write (four 4-byte writes at a lane stride of four words would
+                        // hit every bank four times)
+                        typedef float f4 __attribute__((ext_vector_type(4)));
+                        *reinterpret_cast<f4 *>(__builtin_assume_aligned(q, 16)) =
+                            f4{pre[k].get(0), pre[k].get(1), pre[k].get(2), pre[k].get(3)};
+                    } else {
 #pragma unroll
-                    for (int e = 0; e < VL; e++) q[Map::step(e)] = pre[k].get(e);
+                        for (int e = 0; e < VL; e++) q[Map::step(e)] = pre[k].get(e);
+                    }
                 } else {
 #pragma unroll
                     for (int e = 0; e < VL; e++) {
@@ -258,6 +274,8 @@ struct Stager {
 // (r, w0) to (r, w0 + e) when w0 is a multiple of four and the row is at least four wide.
 template <class G>
 struct GeoMap {
+    // rows whose four-element chunks land on 16-byte boundaries of adjacent words
+    static constexpr bool kWide = G::CLS != CLS_H && G::RS % 4 == 0 && G::PL % 4 == 0;
     static __device__ __forceinline__ unsigned index(int r, int w) {
         return G::interior_row(r) + G::col(w + G::PL);
     }
@@ -296,10 +314,10 @@ constexpr int plan_fma_count(const P &p, int L) {
     return n;
 }
 
-// Workgroup -> (channel, image group).  Hardware hands consecutive workgroup ids to the eight
-// XCDs round-robin and fills the CUs of an XCD in order.  Channels are taken from the tap
-// table's class-cycling order (position p holds a channel of class p mod 8 while all classes
-// last), and the task id is rotated inside every aligned block of eight ids by
+// Workgroup -> (channel, image group) of fprop and dgrad.  Hardware hands consecutive workgroup
+// ids to the eight XCDs round-robin and fills the CUs of an XCD in order.  Channels are taken
+// from the tap table's class-cycling order (position p holds a channel of class p mod 8 while
+// all classes last), and the task id is rotated inside every aligned block of eight ids by
 // (block + block/32), so every XCD and every CU gets a mix of orientations (hence of costs).
 __device__ __forceinline__ void plane_task(const void *blob, int C, int K, int groups, int &c,
                                            int &group) {
@@ -309,6 +327,26 @@ __device__ __forceinline__ void plane_task(const void *blob, int C, int K, int g
     if (j * 8 + 8 <= total) t = (j << 3) + ((i + j + (j >> 5)) & 7);
     c = taps_order(blob, C, K)[t % C];
     group = t / C;
+}
+// Workgroup -> (channel, image group) of wgrad.  Tasks are numbered channel-major over the tap
+// table's class-sorted channel list (a channel's image groups adjacent).  Workgroup ids b,
+// b + cus, b + 2 cus, .. meet on one CU (see above): those get consecutive tasks, i.e. the
+// workgroups that share a CU run the same orientation class, usually the same channel.  With
+// different classes on one CU the wgrad kernel measured 15 % slower at 56 x 56 (fprop and
+// dgrad measured the same or slightly better mixed, hence the two orders).  The host pads grids
+// above `cus` to a multiple of it; returns false for a padding workgroup.
+__device__ __forceinline__ bool wgrad_task(const void *blob, int C, int K, int groups, int cus,
+                                           int &c, int &group) {
+    const int b = blockIdx.x, total = C * groups;
+    int tau = b;
+    if ((int)gridDim.x > cus) {
+        const int q = gridDim.x / cus;
+        tau = (b % cus) * q + b / cus;
+    }
+    if (tau >= total) return false;
+    c = taps_sorted(blob, C, K)[tau / groups];
+    group = tau % groups;
+    return true;
 }
 // Images [n0, n1) of group g: the ceil(N/PB) staged batches are split as evenly as possible.
 template <int PB>
@@ -327,7 +365,14 @@ constexpr int out_tile_offset() {
 }
 template <typename T, int H, int W>
 constexpr bool use_out_tile() {
-    return sizeof(T) < 4 && (H * W) % 4 == 0;  // 4-byte stores run at full rate as they are
+    return (H * W) % 4 == 0;
+}
+// Which classes go through the out-tile: for 16-bit activations both (2-byte stores run far
+// below the rate of wider ones); for fp32 the diagonal class only (its row-shifted 4-byte
+// stores measured 10 % slower than the tile's 16-byte ones, the stacked class's did not).
+template <typename T, int CLS>
+constexpr bool out_tile_class() {
+    return CLS == CLS_D || (CLS == CLS_V && sizeof(T) < 4);
 }
 template <typename T, int H, int W, int PB, int NT>
 __device__ __forceinline__ void flush_out_tile(const float *lout, T *__restrict__ obase,
@@ -460,21 +505,24 @@ __device__ __forceinline__ void run_canonical(const T *__restrict__ src, const f
     const T *sbase = src + (size_t)c * (H * W);
     T *dbase = dst + (size_t)c * (H * W);
 
-    constexpr bool TILE = G::CLS != CLS_H && use_out_tile<T, H, W>();
+    constexpr bool TILE = out_tile_class<T, G::CLS>() && use_out_tile<T, H, W>();
     float *lout = lds + out_tile_offset<K, H, W>();
 
     // Two register sets keep two batches in flight from HBM while a third is being computed.
     auto process = [&](auto &stg, int nb) {
         const int nvalid = n1 - nb;
         __syncthreads();  // previous batch fully consumed (first pass: zero fill done)
-        if constexpr (TILE) {
-            if (nb > n0)
-                flush_out_tile<T, H, W, PB, NT>(lout, dbase + (size_t)(nb - PB) * pstride, pstride, PB);
-        }
         if constexpr (PAIR)
             stg.template commit_pairs<GeoMap<G>, PLS, G::EH, G::EW>(lds, nvalid);
         else
             stg.template commit<GeoMap<G>, PLS>(lds, nvalid);
+        // The previous batch's results leave after the commit: the commit waits for every
+        // outstanding global access of the wave, and stores issued just before it would make
+        // it wait for their acknowledgement too.
+        if constexpr (TILE) {
+            if (nb > n0)
+                flush_out_tile<T, H, W, PB, NT>(lout, dbase + (size_t)(nb - PB) * pstride, pstride, PB);
+        }
         __syncthreads();
         if (nb + 2 * PB < n1)
             stg.prefetch(sbase + (size_t)(nb + 2 * PB) * pstride, pstride, n1 - nb - 2 * PB);
@@ -550,6 +598,7 @@ struct TableMap {
     static constexpr int PAD = table_pad<K, H, W>();
     static constexpr int PL = (PAD + 3) & ~3;
     static constexpr int RS = W + PL + PAD;
+    static constexpr bool kWide = RS % 4 == 0;
     static __device__ __forceinline__ unsigned index(unsigned r, unsigned w) {
         return (r + PAD) * RS + w + PL;
     }
@@ -638,8 +687,12 @@ __device__ __forceinline__ float wave_sum_dpp(float v) {
 struct WgradOut {
     float *part, *dw, *db;
     int NG;
+    unsigned *tickets;  // one zeroed counter per channel block, or null: separate reduction pass
     __device__ __forceinline__ void put(int c, int s, int group, int K, float t) const {
-        if (NG > 1)
+        if (NG > 1 && tickets != nullptr)  // read by another workgroup of this launch: see wgrad_finish
+            __hip_atomic_store(part + ((size_t)c * (K + 1) + s) * NG + group, t, __ATOMIC_RELAXED,
+                               __HIP_MEMORY_SCOPE_AGENT);
+        else if (NG > 1)
             part[((size_t)c * (K + 1) + s) * NG + group] = t;
         else if (s < K)
             dw[(size_t)c * K + s] = t;
@@ -647,6 +700,53 @@ struct WgradOut {
             db[c] = t;
     }
 };
+
+// The single cross-workgroup reduction, folded into stage 1: the workgroups of a channel block
+// (channels [c_first, c_first + nch)) each take a ticket after their partials are visible
+// device-wide; the one that draws the last ticket adds the NG partials of every (channel, tap)
+// in index order -- the same fixed order whichever workgroup happens to be last, so the result
+// is bit-reproducible -- writes dw / db and puts the counter back to zero for the next launch.
+// All threads of the workgroup call this (it contains barriers).
+template <int K>
+__device__ __forceinline__ void wgrad_finish(const WgradOut &out, float *lds, int ticket,
+                                             int c_first, int nch) {
+    if (out.NG <= 1 || out.tickets == nullptr) return;  // uniform
+    // Partial sums are written and read with device-scope (cache-bypassing) accesses and the
+    // ticket is a device-scope atomic, all relaxed: a fence pair at device scope would write
+    // back and invalidate the XCD's whole L2 once per workgroup (measured: +20 to +70 % kernel
+    // time).  Order is kept by completion instead: every thread waits until its stores are
+    // acknowledged before the barrier that precedes the ticket, and the last workgroup's loads
+    // are issued only after its ticket value has come back.
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    unsigned *flag = reinterpret_cast<unsigned *>(lds);
+    if (threadIdx.x == 0)
+        *flag = __hip_atomic_fetch_add(out.tickets + ticket, 1u, __ATOMIC_RELAXED,
+                                       __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    if (*flag != (unsigned)out.NG - 1) return;
+    const int NG = out.NG;
+    for (int i = threadIdx.x; i < nch * (K + 1); i += blockDim.x) {
+        const int c = c_first + i / (K + 1), s = i % (K + 1);
+        if (s == K && out.db == nullptr) continue;
+        // (device-scope loads: the other workgroups ran on other XCDs, behind other L2s)
+        const float *p = out.part + ((size_t)c * (K + 1) + s) * NG;
+        auto ld = [&](int g) {
+            return __hip_atomic_load(p + g, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        };
+        float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+        int g = 0;
+        for (; g + 4 <= NG; g += 4) a0 += ld(g), a1 += ld(g + 1), a2 += ld(g + 2), a3 += ld(g + 3);
+        for (; g < NG; g++) a0 += ld(g);
+        const float total = (a0 + a1) + (a2 + a3);
+        if (s == K)
+            out.db[c] = total;
+        else
+            out.dw[(size_t)c * K + s] = total;
+    }
+    if (threadIdx.x == 0)
+        __hip_atomic_store(out.tickets + ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
 
 template <int K, int NT, class SlotOf>
 __device__ __forceinline__ void wgrad_epilogue(float (&acc)[K + 1], float *lds, const WgradOut &out,
@@ -666,14 +766,34 @@ __device__ __forceinline__ void wgrad_epilogue(float (&acc)[K + 1], float *lds, 
             for (int w = 0; w < NW; w++) t += lds[w * (K + 1) + slot];
         out.put(c, threadIdx.x, group, K, t);
     }
+    wgrad_finish<K>(out, lds, c, c, 1);
 }
 
-// dy planes are staged unpadded right behind the x planes and the tap tables
-template <int H, int W>
-struct FlatMap {
-    static __device__ __forceinline__ unsigned index(unsigned r, unsigned w) { return r * W + w; }
+// dy planes are staged without a halo right behind the x planes and the tap tables, rows DRS
+// words apart.  An item reads the dy of its L outputs; for the stacked and diagonal classes
+// that is one word per lane and row, lanes along j, and DRS is chosen like the x rows' stride so
+// that stepping to the next row-block continues the same line modulo the 32 banks.  The
+// row-direction classes read their L adjacent outputs as one wide word: rows stay W apart.
+template <int W, int DRS>
+struct DyMap {
+    static constexpr bool kWide = DRS % 4 == 0;
+    static __device__ __forceinline__ unsigned index(unsigned r, unsigned w) { return r * DRS + w; }
     static constexpr int step(int e) { return e; }
 };
+template <class G, int W>
+constexpr int dy_row_stride() {
+    return G::CLS == CLS_H ? W : bank_stride(W, G::LR, G::IPR);
+}
+template <int K, int H, int W, int... Os>
+constexpr int max_dy_plane(std::integer_sequence<int, Os...>) {
+    int m = H * W;  // table-driven body and row-direction classes
+    ((m = cmax(m, H * dy_row_stride<Geo<Os, K, tile_L<H, W>(Os), H, W>, W>())), ...);
+    return (m + 3) & ~3;
+}
+template <int K, int H, int W>
+constexpr int wgrad_dy_plane() {
+    return max_dy_plane<K, H, W>(std::make_integer_sequence<int, 8>{});
+}
 template <int K, int H, int W>
 constexpr int wgrad_dy_offset() {
     return (Tile<H, W>::PB * plane_floats<K, H, W>() + 2 * K + 3) & ~3;
@@ -694,23 +814,30 @@ __device__ __forceinline__ void run_canonical_wgrad(const T *__restrict__ x, con
     const T *xbase = x + (size_t)c * (H * W);
     const T *gbase = dy + (size_t)c * (H * W);
     float *ldy = lds + wgrad_dy_offset<K, H, W>();
+    constexpr int DRS = dy_row_stride<G, W>(), DYP = wgrad_dy_plane<K, H, W>();
 
     float acc[K + 1];  // acc[s] for representative taps s, acc[K] = sum of dy (bias gradient)
 #pragma unroll
     for (int s = 0; s <= K; s++) acc[s] = 0.f;
 
-    Stager<T, H, W, PB, NT> sx, sg;
-    sx.prefetch(xbase + (size_t)n0 * pstride, pstride, n1 - n0);
-    sg.prefetch(gbase + (size_t)n0 * pstride, pstride, n1 - n0);
-    for (int nb = n0; nb < n1; nb += PB) {
+    // Two register sets per tensor keep two batches in flight while a third is being summed.
+    constexpr int DEPTH = DWO_WGRAD_DEPTH;
+    Stager<T, H, W, PB, NT> sx[DEPTH], sg[DEPTH];
+#pragma unroll
+    for (int k = 0; k < DEPTH; k++)
+        if (n0 + k * PB < n1) {
+            sx[k].prefetch(xbase + (size_t)(n0 + k * PB) * pstride, pstride, n1 - n0 - k * PB);
+            sg[k].prefetch(gbase + (size_t)(n0 + k * PB) * pstride, pstride, n1 - n0 - k * PB);
+        }
+    auto process = [&](auto &stx, auto &stg, int nb) {
         const int nvalid = n1 - nb;
         __syncthreads();
-        sx.template commit<GeoMap<G>, PLS>(lds, nvalid);
-        sg.template commit<FlatMap<H, W>, H * W>(ldy, nvalid);
+        stx.template commit<GeoMap<G>, PLS>(lds, nvalid);
+        stg.template commit<DyMap<W, DRS>, DYP>(ldy, nvalid);
         __syncthreads();
-        if (nb + PB < n1) {
-            sx.prefetch(xbase + (size_t)(nb + PB) * pstride, pstride, nvalid - PB);
-            sg.prefetch(gbase + (size_t)(nb + PB) * pstride, pstride, nvalid - PB);
+        if (nb + DEPTH * PB < n1) {
+            stx.prefetch(xbase + (size_t)(nb + DEPTH * PB) * pstride, pstride, nvalid - DEPTH * PB);
+            stg.prefetch(gbase + (size_t)(nb + DEPTH * PB) * pstride, pstride, nvalid - DEPTH * PB);
         }
 #pragma unroll
         for (int it = 0; it < ITERS; it++) {
@@ -720,7 +847,7 @@ __device__ __forceinline__ void run_canonical_wgrad(const T *__restrict__ x, con
             if (item < PB * G::IPP && (int)pl < nvalid) {
                 // dy of the item's L outputs (zero where the output does not exist)
                 float d[L];
-                const float *g = ldy + pl * (H * W);
+                const float *g = ldy + pl * DYP;
                 if constexpr (G::CLS == CLS_H) {
                     // one wide read: L separate reads at a lane stride of L words conflict L ways
                     if constexpr (L == 4 && W % 4 == 0 && (H * W) % 4 == 0) {
@@ -736,13 +863,13 @@ __device__ __forceinline__ void run_canonical_wgrad(const T *__restrict__ x, con
                 } else if constexpr (G::CLS == CLS_V) {
 #pragma unroll
                     for (int l = 0; l < L; l++)
-                        d[l] = (H % L == 0 || rb * L + l < H) ? g[(rb * L + l) * W + j] : 0.f;
+                        d[l] = (H % L == 0 || rb * L + l < H) ? g[(rb * L + l) * DRS + j] : 0.f;
                 } else {
 #pragma unroll
                     for (int l = 0; l < L; l++) {
                         const unsigned q = j + (unsigned)(l - G::Q0);
                         const bool ok = q < W && (H % L == 0 || rb * L + G::P0 + l * G::EH < H);
-                        d[l] = ok ? g[(int)(rb * (L * W) + j) + (G::P0 + l * G::EH) * W + l - G::Q0] : 0.f;
+                        d[l] = ok ? g[(int)(rb * (L * DRS) + j) + (G::P0 + l * G::EH) * DRS + l - G::Q0] : 0.f;
                     }
                 }
                 const float *base = lds + (pl * PLS + rb * (G::LR * G::RS) + j);
@@ -759,6 +886,11 @@ __device__ __forceinline__ void run_canonical_wgrad(const T *__restrict__ x, con
                 for (int l = 0; l < L; l++) acc[K] += d[l];
             }
         }
+    };
+    for (int nb = n0; nb < n1; nb += DEPTH * PB) {
+        process(sx[0], sg[0], nb);
+        if constexpr (DEPTH > 1)
+            if (nb + PB < n1) process(sx[DEPTH - 1], sg[DEPTH - 1], nb + PB);
     }
     wgrad_epilogue<K, NT>(acc, lds, out, c, group, [](int s) { return (int)G::plan.rep[s]; });
 }
@@ -816,11 +948,11 @@ __device__ __forceinline__ void run_table_wgrad(const T *__restrict__ x, const T
 template <typename T, int K, int H, int W>
 __global__ __launch_bounds__((Tile<H, W>::NT)) __attribute__((amdgpu_waves_per_eu(DWO_WPE_WGRAD, 8))) void plane_wgrad_kernel(
     const T *__restrict__ x, const T *__restrict__ dy, const void *__restrict__ blob,
-    WgradOut out, int N, int C) {
-    extern __shared__ float lds[];
+    WgradOut out, int N, int C, int cus) {
+    extern __shared__ __align__(16) float lds[];
     const int NG = out.NG;
     int c, group;
-    plane_task(blob, C, K, NG, c, group);
+    if (!wgrad_task(blob, C, K, NG, cus, c, group)) return;
     int n0, n1;
     group_range<Tile<H, W>::PB>(N, NG, group, n0, n1);
     const int cls = taps_class(blob, C, K)[c];
@@ -851,14 +983,14 @@ constexpr size_t plane_kernel_lds_bytes() {
 }
 template <int K, int H, int W>
 constexpr size_t plane_wgrad_lds_bytes() {
-    return ((size_t)wgrad_dy_offset<K, H, W>() + Tile<H, W>::PB * H * W) * sizeof(float);
+    return ((size_t)wgrad_dy_offset<K, H, W>() + Tile<H, W>::PB * wgrad_dy_plane<K, H, W>()) * sizeof(float);
 }
 
 template <int OP, typename T, int K, int H, int W>
 __global__ __launch_bounds__((Tile<H, W>::NT)) __attribute__((amdgpu_waves_per_eu(DWO_WPE, 8))) void plane_kernel(
     const T *__restrict__ src, const float *__restrict__ wt, const float *__restrict__ bias,
     const void *__restrict__ blob, T *__restrict__ dst, int N, int C, int groups) {
-    extern __shared__ float lds[];
+    extern __shared__ __align__(16) float lds[];
     int c, group;
     plane_task(blob, C, K, groups, c, group);
     int n0, n1;
@@ -888,16 +1020,22 @@ __global__ __launch_bounds__((Tile<H, W>::NT)) __attribute__((amdgpu_waves_per_e
 // ---------------------------------------------------------------------------------------------
 // host launchers (instantiated per element type and plane extent in dwo_inst.hip)
 // ---------------------------------------------------------------------------------------------
-// Workgroups that can be resident at once on the current device for a kernel.
+// Workgroups that can be resident at once on the current device for a kernel, and the device's
+// CU count, packed as slots | cus << 16.
 template <class Kern>
 int resident_slots(Kern kern, int block, size_t lds) {
     int dev = 0, cus = 0, per_cu = 0;
     if (hipGetDevice(&dev) != hipSuccess ||
         hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
         hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kern, block, lds) != hipSuccess ||
-        cus < 1 || per_cu < 1)
-        return 1024;
-    return cus * per_cu;
+        cus < 1 || per_cu < 1 || cus > 4096 || cus * per_cu > 65535)
+        return 1024 | (256 << 16);
+    return (cus * per_cu) | (cus << 16);
+}
+// grid of C * groups tasks, padded to a multiple of the CU count once it exceeds it (wgrad_task)
+inline unsigned plane_grid(int C, int groups, int cus) {
+    const long total = (long)C * groups;
+    return (unsigned)(total > cus ? (total + cus - 1) / cus * cus : total);
 }
 
 template <typename T, int K, int H, int W>
@@ -906,9 +1044,10 @@ int launch_plane_conv(int op, const void *src, const float *w, const float *bias
     constexpr int NT = Tile<H, W>::NT;
     const size_t lds = plane_kernel_lds_bytes<T, K, H, W>();
     static int cache[kMaxDevices];
-    const int slots_f = per_device_once(
+    const int packed = per_device_once(
         cache, [&] { return resident_slots(plane_kernel<OP_FPROP, T, K, H, W>, NT, lds); });
     if (N == 0) return 0;  // set-up only
+    const int slots_f = packed & 0xffff;
     const int groups = plane_groups(N, C, Tile<H, W>::PB, slots_f);
     const dim3 grid(C * groups), block(NT);
     if (op == OP_FPROP)
@@ -922,20 +1061,22 @@ int launch_plane_conv(int op, const void *src, const float *w, const float *bias
 }
 
 // Writes NG = *groups_out partials per (channel, tap) into part[(c*(K+1)+s)*NG + g]; with
-// NG = 1 the sums go straight to dw / db (db may be null) and no reduction is needed.
+// NG = 1 the sums go straight to dw / db (db may be null) and no reduction is needed, and with
+// `tickets` (C zeroed counters) the last workgroup of each channel reduces them itself.
 template <typename T, int K, int H, int W>
 int launch_plane_wgrad(const void *x, const void *dy, const void *taps, float *part, float *dw,
-                       float *db, int N, int C, int *groups_out, hipStream_t st) {
+                       float *db, unsigned *tickets, int N, int C, int *groups_out, hipStream_t st) {
     constexpr int NT = Tile<H, W>::NT;
     const size_t lds = plane_wgrad_lds_bytes<K, H, W>();
     static int cache[kMaxDevices];
-    const int slots = per_device_once(
+    const int packed = per_device_once(
         cache, [&] { return resident_slots(plane_wgrad_kernel<T, K, H, W>, NT, lds); });
     if (N == 0) return 0;  // set-up only
+    const int slots = packed & 0xffff, cus = packed >> 16;
     const int groups = plane_groups(N, C, Tile<H, W>::PB, slots);
     *groups_out = groups;
-    plane_wgrad_kernel<T, K, H, W><<<dim3(C * groups), dim3(NT), lds, st>>>(
-        (const T *)x, (const T *)dy, taps, WgradOut{part, dw, db, groups}, N, C);
+    plane_wgrad_kernel<T, K, H, W><<<dim3(plane_grid(C, groups, cus)), dim3(NT), lds, st>>>(
+        (const T *)x, (const T *)dy, taps, WgradOut{part, dw, db, groups, tickets}, N, C, cus);
     const hipError_t e = hipGetLastError();
     return e == hipSuccess ? 0 : (int)e;
 }
