@@ -2,6 +2,7 @@
 //   -DDWO_INST_T=<float|bf16_t|f16_t> -DDWO_INST_K=<K> -DDWO_INST_H=<H> -DDWO_INST_W=<W>
 #include "dwo_static.h"
 #include "dwo_nhwc_plane.h"
+#include "dwo_regplane.h"
 
 namespace dwo {
 template int launch_plane_conv<DWO_INST_T, DWO_INST_K, DWO_INST_H, DWO_INST_W>(

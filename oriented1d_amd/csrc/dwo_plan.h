@@ -274,6 +274,14 @@ constexpr int tile_L(int o) {
                                     : (orient_class(o) == CLS_V ? Tile<H, W>::LV : Tile<H, W>::LD);
 }
 
+// Planes of at most 16 x 16 are handled in registers, one plane per 16-lane DPP row
+// (dwo_regplane.h), instead of being staged in LDS.
+constexpr bool reg_plane_shape_rt(int H, int W) { return H <= 16 && W <= 16; }
+template <int H, int W>
+constexpr bool reg_plane_shape() {
+    return reg_plane_shape_rt(H, W);
+}
+
 // NHWC slice kernels: a workgroup owns kSliceCh consecutive channels.
 constexpr int kSliceCh = 4;
 // Threads per workgroup and images staged per batch: the planes of a batch must fit in LDS, and

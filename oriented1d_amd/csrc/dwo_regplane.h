@@ -1,0 +1,294 @@
+// Register-plane NCHW fprop / dgrad kernels for stride 1 on planes of at most 16 x 16 (the
+// 14 x 14 and 7 x 7 stages): no barriers, LDS only as a wave-private turntable between the
+// coalesced global accesses and the lanes' rows.  (wgrad of these planes stays on the LDS-staged
+// plane kernels: its 32 running sums next to two planes in registers did not fit without
+// spilling, and measured slower.)
+//
+// A plane lives in the registers of one 16-lane DPP row: lane i of the row holds row i of the
+// plane (W registers) for the row-direction and diagonal orientations, or column i (H registers)
+// for the stacked ones.  A tap (dh, dw) then is a compile-time register index (the offset along
+// the registers) plus a DPP row shift by the offset across the lanes, applied as a modifier of
+// the multiply-add's source operand: lanes shifted in from outside the 16-lane row read zero
+// (bound_ctrl), which is exactly the operator's out-of-image rule, and the unused lanes of a row
+// hold zeros.  A wave works on four planes (images n .. n+3 of one channel); the waves of a
+// workgroup take consecutive channels of the same images, so a workgroup reads and writes one
+// contiguous run of memory per image (whole cache lines when the channel block starts on one),
+// each wave running the body of its own channel's orientation.
+#pragma once
+
+#include "dwo_common.h"
+#include "dwo_dispatch.h"
+#include "dwo_plan.h"
+#include "dwo_static.h"
+
+namespace dwo {
+
+constexpr int kRegPlanesPerWave = 4;   // one per 16-lane DPP row
+constexpr int kRegWavesPerGroup = 8;   // consecutive channels per workgroup
+constexpr int kRegThreads = 64 * kRegWavesPerGroup;
+
+// lanes hold rows for the row-direction and diagonal classes, columns for the stacked ones
+constexpr bool reg_lane_is_row(int o) { return orient_class(o) != CLS_V; }
+
+// value of `v` in lane (own lane + SH) of the same 16-lane row, zero beyond the row
+template <int SH>
+__device__ __forceinline__ float row_shift(float v) {
+    if constexpr (SH == 0) {
+        return v;
+    } else {
+        constexpr int ctrl = SH > 0 ? 0x100 + SH : 0x110 - SH;  // row_shl:SH / row_shr:-SH
+        return __builtin_bit_cast(
+            float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), ctrl, 0xf, 0xf, true));
+    }
+}
+
+// taps of orientation O on an H x W plane: rep[s] = first tap with the same offset (duplicates
+// fold into it), -1 for a tap that cannot reach the plane
+template <int O, int K, int H, int W>
+struct RegPlan {
+    static constexpr Plan plan = make_plan(O, K, 1, H, W);
+};
+
+// does any live, representative tap of orientation O shift by SH lanes?
+template <int O, int K, int H, int W>
+constexpr bool reg_shift_used(int sh) {
+    for (int s = 0; s < K; s++)
+        if (RegPlan<O, K, H, W>::plan.rep[s] == s &&
+            (reg_lane_is_row(O) ? canon_dh(O, K, s) : canon_dw(O, K, s)) == sh)
+            return true;
+    return false;
+}
+
+// The four planes of a wave travel between HBM and the registers through a wave-private piece
+// of LDS (fp32, planes back to back, no halo): global accesses are whole 16-byte (8-byte for
+// 16-bit types) chunks at consecutive addresses from consecutive lanes, whatever way the lanes
+// then pick their rows or columns out of LDS.  (Rows fetched from HBM directly, 56 bytes apart
+// from lane to lane, ran 1.7 times slower at 14 x 14.)  Only one wave touches the region and a
+// wave's LDS operations complete in order, so no barrier is involved.
+template <typename T, int H, int W>
+struct RegIO {
+    static constexpr int E = H * W, VL = E % 4 == 0 ? 4 : 1;
+    static constexpr int NCH = E / VL, NIT = (NCH + 63) / 64;
+    static constexpr int kWaveFloats = kRegPlanesPerWave * E;
+    Chunk<T, VL> reg[kRegPlanesPerWave][NIT];
+
+    // base = plane (n0, c); planes n0 .. n0+nvalid-1 exist, `stride` elements apart
+    __device__ __forceinline__ void fetch(const T *__restrict__ base, size_t stride, int nvalid) {
+        const unsigned lane = threadIdx.x & 63;
+#pragma unroll
+        for (int p = 0; p < kRegPlanesPerWave; p++)
+#pragma unroll
+            for (int it = 0; it < NIT; it++) {
+                const unsigned l = lane + 64 * it;
+                if (l < NCH && p < nvalid) reg[p][it].load(base + p * stride + l * VL);
+            }
+    }
+    __device__ __forceinline__ void put(float *wl, int nvalid) const {
+        const unsigned lane = threadIdx.x & 63;
+#pragma unroll
+        for (int p = 0; p < kRegPlanesPerWave; p++)
+#pragma unroll
+            for (int it = 0; it < NIT; it++) {
+                const unsigned l = lane + 64 * it;
+                if (l < NCH && p < nvalid) {
+                    float *q = wl + p * E + l * VL;
+                    if constexpr (VL == 4) {
+                        typedef float f4 __attribute__((ext_vector_type(4)));
+                        *reinterpret_cast<f4 *>(__builtin_assume_aligned(q, 16)) =
+                            f4{reg[p][it].get(0), reg[p][it].get(1), reg[p][it].get(2),
+                               reg[p][it].get(3)};
+                    } else {
+                        q[0] = reg[p][it].get(0);
+                    }
+                }
+            }
+        __builtin_amdgcn_wave_barrier();
+    }
+    // results in the wave's LDS region -> HBM
+    static __device__ __forceinline__ void write_out(const float *wl, T *__restrict__ base,
+                                                     size_t stride, int nvalid) {
+        __builtin_amdgcn_wave_barrier();
+        const unsigned lane = threadIdx.x & 63;
+#pragma unroll
+        for (int p = 0; p < kRegPlanesPerWave; p++)
+#pragma unroll
+            for (int it = 0; it < NIT; it++) {
+                const unsigned l = lane + 64 * it;
+                if (l < NCH && p < nvalid) {
+                    const float *q = wl + p * E + l * VL;
+                    if constexpr (VL == 4) {
+                        const float4 v = *reinterpret_cast<const float4 *>(__builtin_assume_aligned(q, 16));
+                        Vec4<T> r;
+                        r.set(v.x, v.y, v.z, v.w);
+                        r.store(base + p * stride + l * VL);
+                    } else {
+                        st_out(base + p * stride + l, from_float<T>(q[0]));
+                    }
+                }
+            }
+    }
+};
+
+// A plane in registers: lane i of 16-lane row `ps` holds row i (ROW) or column i of plane ps.
+template <bool ROW, int H, int W>
+struct RegPlane {
+    static constexpr int NREG = ROW ? W : H, NLANE = ROW ? H : W;
+    float v[NREG];
+    // wl = the wave's LDS region; lanes beyond the plane (and the rows of missing planes) hold zeros
+    __device__ __forceinline__ void load(const float *wl, unsigned ps, unsigned i, bool plane_ok) {
+        const bool live = plane_ok && i < NLANE;
+        const float *p = wl + ps * (H * W) + (ROW ? i * W : i);
+#pragma unroll
+        for (int q = 0; q < NREG; q++) v[q] = live ? p[ROW ? q : q * W] : 0.f;
+    }
+    __device__ __forceinline__ void store(float *wl, unsigned ps, unsigned i, bool plane_ok) const {
+        const bool live = plane_ok && i < NLANE;
+        float *p = wl + ps * (H * W) + (ROW ? i * W : i);
+        if (live) {
+#pragma unroll
+            for (int q = 0; q < NREG; q++) p[ROW ? q : q * W] = v[q];
+        }
+    }
+};
+
+// ---------------------------------------------------------------------------------------------
+// fprop / dgrad
+// ---------------------------------------------------------------------------------------------
+template <int O, int OP, typename T, int K, int H, int W>
+__device__ __forceinline__ void regplane_conv_body(const T *__restrict__ src,
+                                                   const float *__restrict__ wt,
+                                                   const float *__restrict__ bias,
+                                                   T *__restrict__ dst, float *wl, int c, int C,
+                                                   int n0, int N) {
+    constexpr bool ROW = reg_lane_is_row(O);
+    using P = RegPlane<ROW, H, W>;
+    using IO = RegIO<T, H, W>;
+    constexpr int NREG = P::NREG;
+    using RP = RegPlan<O, K, H, W>;  // rep[]: duplicate and dead taps
+    const unsigned lane = threadIdx.x & 63, i = lane & 15, ps = lane >> 4;
+    const size_t off = ((size_t)n0 * C + c) * (H * W), stride = (size_t)C * (H * W);
+    const int nvalid = N - n0;  // planes of this wave that exist (may exceed four)
+    IO io;
+    io.fetch(src + off, stride, nvalid);
+
+    // weights with duplicates folded into their representative tap (dgrad: reversed, the
+    // offsets are odd-symmetric)
+    float w[K];
+#pragma unroll
+    for (int s = 0; s < K; s++) w[s] = wt[(size_t)c * K + (OP == OP_DGRAD ? K - 1 - s : s)];
+    static_for<K>([&](auto s) {
+        constexpr int r = RP::plan.rep[s];
+        if constexpr (r >= 0 && r != s) w[r] += w[s];
+    });
+    const float bv = (OP == OP_FPROP && bias != nullptr) ? bias[c] : 0.f;
+    io.put(wl, nvalid);
+    P x;
+    x.load(wl, ps, i, (int)ps < nvalid);
+    // Shift by shift: the plane shifted by SH lanes (one DPP move per register), then every
+    // multiply-add whose tap has that shift.  The empty asm at the end of a shift pins the
+    // running sums there, so the shifted copies die with their shift (left to itself the
+    // compiler makes the copies of all shifts first and spills them).
+    P y;
+#pragma unroll
+    for (int q = 0; q < NREG; q++) y.v[q] = bv;
+    static_for<31>([&](auto idx) {
+        constexpr int sh = idx - 15;
+        if constexpr (reg_shift_used<O, K, H, W>(sh)) {
+            float xs[NREG];
+#pragma unroll
+            for (int j = 0; j < NREG; j++) xs[j] = row_shift<sh>(x.v[j]);
+            static_for<K>([&](auto s) {
+                if constexpr (RP::plan.rep[s] == s && (ROW ? canon_dh(O, K, s) : canon_dw(O, K, s)) == sh) {
+                    constexpr int o = ROW ? canon_dw(O, K, s) : canon_dh(O, K, s);
+                    static_for<NREG>([&](auto q) {
+                        constexpr int j = q + o;
+                        if constexpr (j >= 0 && j < NREG) y.v[q] = __builtin_fmaf(xs[j], w[s], y.v[q]);
+                    });
+                }
+            });
+#pragma unroll
+            for (int q = 0; q < NREG; q++) asm volatile("" : "+v"(y.v[q]));
+        }
+    });
+    y.store(wl, ps, i, (int)ps < nvalid);
+    IO::write_out(wl, dst + off, stride, nvalid);
+}
+
+// any angle: every output gathers its taps from global memory through the caches (rare: the
+// networks only use the canonical orientations)
+template <int OP, typename T, int K, int H, int W>
+__device__ __forceinline__ void regplane_conv_table(const T *__restrict__ src,
+                                                    const float *__restrict__ wt,
+                                                    const float *__restrict__ bias,
+                                                    const int8_t *__restrict__ dhdw,
+                                                    T *__restrict__ dst, int c, int C, int n0, int N) {
+    const unsigned lane = threadIdx.x & 63, i = lane & 15;
+    const int n = n0 + (int)(lane >> 4);
+    if (n >= N || i >= H) return;
+    const size_t off = ((size_t)n * C + c) * (H * W);
+    const float bv = (OP == OP_FPROP && bias != nullptr) ? bias[c] : 0.f;
+    for (int q = 0; q < W; q++) {
+        float acc = bv;
+        for (int s = 0; s < K; s++) {
+            const int sgn = OP == OP_DGRAD ? -1 : 1;
+            const int h = (int)i + sgn * dhdw[((size_t)c * K + s) * 2];
+            const int ww = q + sgn * dhdw[((size_t)c * K + s) * 2 + 1];
+            if (h >= 0 && h < H && ww >= 0 && ww < W)
+                acc = __builtin_fmaf(to_float(src[off + h * W + ww]), wt[(size_t)c * K + s], acc);
+        }
+        st_out(dst + off + i * W + q, from_float<T>(acc));
+    }
+}
+
+template <int OP, typename T, int K, int H, int W>
+__global__ __launch_bounds__(kRegThreads) __attribute__((amdgpu_waves_per_eu(6, 8))) void regplane_kernel(
+    const T *__restrict__ src, const float *__restrict__ wt, const float *__restrict__ bias,
+    const void *__restrict__ blob, T *__restrict__ dst, int N, int C) {
+    // (wave-uniform: the weights and the class are fetched with scalar loads)
+    const int c = blockIdx.x * kRegWavesPerGroup + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    if (c >= C) return;  // whole wave; the kernel has no barriers
+    __shared__ __align__(16) float lds[kRegWavesPerGroup * RegIO<T, H, W>::kWaveFloats];
+    float *wl = lds + (threadIdx.x >> 6) * RegIO<T, H, W>::kWaveFloats;
+    const int n0 = blockIdx.y * kRegPlanesPerWave;
+    const int cls = __builtin_amdgcn_readfirstlane(taps_class(blob, C, K)[c]);
+#define DWO_CASE(O)                                                             \
+    case O:                                                                     \
+        regplane_conv_body<O, OP, T, K, H, W>(src, wt, bias, dst, wl, c, C, n0, N); \
+        break;
+    switch (cls) {
+        DWO_CASE(0)
+        DWO_CASE(1)
+        DWO_CASE(2)
+        DWO_CASE(3)
+        DWO_CASE(4)
+        DWO_CASE(5)
+        DWO_CASE(6)
+        DWO_CASE(7)
+        default:
+            regplane_conv_table<OP, T, K, H, W>(src, wt, bias, taps_dhdw(blob), dst, c, C, n0, N);
+    }
+#undef DWO_CASE
+}
+
+// ---------------------------------------------------------------------------------------------
+// host launcher (same contract as launch_plane_conv)
+// ---------------------------------------------------------------------------------------------
+template <typename T, int K, int H, int W>
+int launch_regplane_conv(int op, const void *src, const float *w, const float *bias,
+                         const void *taps, void *dst, int N, int C, hipStream_t st) {
+    if (N == 0) return 0;  // set-up only: nothing to prepare
+    const dim3 grid((C + kRegWavesPerGroup - 1) / kRegWavesPerGroup,
+                    (N + kRegPlanesPerWave - 1) / kRegPlanesPerWave),
+        block(kRegThreads);
+    if (grid.y > 65535) return DWO_ERR_BAD_SHAPE;
+    if (op == OP_FPROP)
+        regplane_kernel<OP_FPROP, T, K, H, W><<<grid, block, 0, st>>>((const T *)src, w, bias, taps,
+                                                                     (T *)dst, N, C);
+    else
+        regplane_kernel<OP_DGRAD, T, K, H, W><<<grid, block, 0, st>>>((const T *)src, w, bias, taps,
+                                                                     (T *)dst, N, C);
+    const hipError_t e = hipGetLastError();
+    return e == hipSuccess ? 0 : (int)e;
+}
+
+}  // namespace dwo

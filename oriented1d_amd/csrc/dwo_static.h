@@ -1038,9 +1038,16 @@ inline unsigned plane_grid(int C, int groups, int cus) {
     return (unsigned)(total > cus ? (total + cus - 1) / cus * cus : total);
 }
 
+// register-plane kernels (dwo_regplane.h) take fprop and dgrad of planes of at most 16 x 16
+template <typename T, int K, int H, int W>
+int launch_regplane_conv(int op, const void *src, const float *w, const float *bias,
+                         const void *taps, void *dst, int N, int C, hipStream_t st);
 template <typename T, int K, int H, int W>
 int launch_plane_conv(int op, const void *src, const float *w, const float *bias, const void *taps,
                       void *dst, int N, int C, hipStream_t st) {
+    if constexpr (reg_plane_shape<H, W>()) {
+        return launch_regplane_conv<T, K, H, W>(op, src, w, bias, taps, dst, N, C, st);
+    } else {
     constexpr int NT = Tile<H, W>::NT;
     const size_t lds = plane_kernel_lds_bytes<T, K, H, W>();
     static int cache[kMaxDevices];
@@ -1058,6 +1065,7 @@ int launch_plane_conv(int op, const void *src, const float *w, const float *bias
                                                                    (T *)dst, N, C, groups);
     const hipError_t e = hipGetLastError();
     return e == hipSuccess ? 0 : (int)e;
+    }
 }
 
 // Writes NG = *groups_out partials per (channel, tap) into part[(c*(K+1)+s)*NG + g]; with
