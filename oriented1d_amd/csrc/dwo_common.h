@@ -8,6 +8,19 @@
 
 namespace dwo {
 
+// One 16-byte (8-byte) LDS read of four (two) adjacent words; p must be aligned to the access.
+// A float4 / float2 dereference is taken apart into 4-byte reads by the passes this library
+// is built with; at a lane stride of four words those hit every bank eight times.
+typedef float lds_f4 __attribute__((ext_vector_type(4)));
+typedef float lds_f2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ lds_f4 lds_read4(const float *p) {
+    return *reinterpret_cast<const lds_f4 *>(__builtin_assume_aligned(p, 16));
+}
+__device__ __forceinline__ lds_f2 lds_read2(const float *p) {
+    return *reinterpret_cast<const lds_f2 *>(__builtin_assume_aligned(p, 8));
+}
+
+
 // ---------------------------------------------------------------------------------------------
 // Tap blob (private layout).  Built on the host by dwo_build_taps, copied verbatim to the device.
 //   int32 header[8] : magic, version, C, K, off_dhdw, off_class, off_order, off_extent

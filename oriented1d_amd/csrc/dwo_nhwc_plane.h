@@ -490,11 +490,11 @@ __device__ __forceinline__ void nhwc_canonical_wgrad(NhwcWgradCtx<T, K, H, W> &c
                     if constexpr (G::CLS == CLS_H) {
                         // one wide read: L separate reads at a lane stride of L words conflict L ways
                         if constexpr (L == 4 && W % 4 == 0) {
-                            const float4 dv = *reinterpret_cast<const float4 *>(g + rb * W + j * 4);
-                            d[0] = dv.x, d[1] = dv.y, d[2] = dv.z, d[3] = dv.w;
+                            const lds_f4 dv = lds_read4(g + rb * W + j * 4);
+                            d[0] = dv[0], d[1] = dv[1], d[2] = dv[2], d[3] = dv[3];
                         } else if constexpr (L == 2 && W % 2 == 0) {
-                            const float2 dv = *reinterpret_cast<const float2 *>(g + rb * W + j * 2);
-                            d[0] = dv.x, d[1] = dv.y;
+                            const lds_f2 dv = lds_read2(g + rb * W + j * 2);
+                            d[0] = dv[0], d[1] = dv[1];
                         } else {
 #pragma unroll
                             for (int l = 0; l < L; l++) d[l] = g[rb * W + j * L + l];

@@ -1,6 +1,7 @@
 // Register-plane NCHW fprop / dgrad kernels for stride 1 on planes of at most 16 x 16 (the
-// 14 x 14 and 7 x 7 stages): no barriers, LDS only as a wave-private turntable between the
-// coalesced global accesses and the lanes' rows.  (wgrad of these planes stays on the LDS-staged
+// 14 x 14 and 7 x 7 stages): LDS only as a turntable between the coalesced global accesses and
+// the lanes' rows (wave-private and without barriers where a plane is a whole number of
+// four-element chunks).  (wgrad of these planes stays on the LDS-staged
 // plane kernels: its 32 running sums next to two planes in registers did not fit without
 // spilling, and measured slower.)
 //
@@ -117,15 +118,62 @@ struct RegIO {
                 if (l < NCH && p < nvalid) {
                     const float *q = wl + p * E + l * VL;
                     if constexpr (VL == 4) {
-                        const float4 v = *reinterpret_cast<const float4 *>(__builtin_assume_aligned(q, 16));
+                        const lds_f4 v = lds_read4(q);
                         Vec4<T> r;
-                        r.set(v.x, v.y, v.z, v.w);
+                        r.set(v[0], v[1], v[2], v[3]);
                         r.store(base + p * stride + l * VL);
                     } else {
                         st_out(base + p * stride + l, from_float<T>(q[0]));
                     }
                 }
             }
+    }
+};
+
+// Planes whose size is not a multiple of four elements (7 x 7) travel as single elements per
+// lane.  For 16-bit activations those 2-byte accesses cost more than two workgroup barriers
+// (7 x 7 bf16: 9.3 us per launch against 7.2 us; fp32 measured 4 % slower this way and keeps the
+// barrier-free path): when the channel count is a multiple of the workgroup's eight channels,
+// the eight planes of one image are one contiguous, aligned run of 8 * H * W elements, and the
+// workgroup moves the runs of its four images as whole four-element chunks, one per thread,
+// through all the waves' LDS regions.
+template <typename T, int H, int W>
+struct GroupIO {
+    static constexpr int E = H * W;
+    static constexpr bool kUse = E % 4 != 0 && sizeof(T) == 2;  // (8 * E is a multiple of four)
+    static constexpr int RUN = kRegWavesPerGroup * E / 4;      // chunks per image
+    static constexpr int kWaveFloats = kRegPlanesPerWave * E;
+    static_assert(!kUse || kRegPlanesPerWave * RUN <= kRegThreads, "one chunk per thread");
+    Vec4<T> reg;
+
+    // LDS index of element `idx` of image p's run: channel idx / E, element idx % E
+    static __device__ __forceinline__ unsigned slot(unsigned p, unsigned idx) {
+        const unsigned w = idx / E;
+        return w * kWaveFloats + p * E + (idx - w * E);
+    }
+    // base = plane (n0, c0) of the workgroup's first channel
+    __device__ __forceinline__ void fetch(const T *__restrict__ base, size_t stride, int nvalid) {
+        const unsigned p = threadIdx.x / RUN, i = threadIdx.x % RUN;
+        if (p < kRegPlanesPerWave && (int)p < nvalid) reg.load(base + p * stride + i * 4);
+    }
+    __device__ __forceinline__ void put(float *lds, int nvalid) const {
+        const unsigned p = threadIdx.x / RUN, i = threadIdx.x % RUN;
+        if (p < kRegPlanesPerWave && (int)p < nvalid) {
+#pragma unroll
+            for (int e = 0; e < 4; e++) lds[slot(p, i * 4 + e)] = reg.get(e);
+        }
+        __syncthreads();
+    }
+    static __device__ __forceinline__ void write_out(const float *lds, T *__restrict__ base,
+                                                     size_t stride, int nvalid) {
+        __syncthreads();
+        const unsigned p = threadIdx.x / RUN, i = threadIdx.x % RUN;
+        if (p < kRegPlanesPerWave && (int)p < nvalid) {
+            Vec4<T> r;
+            r.set(lds[slot(p, i * 4)], lds[slot(p, i * 4 + 1)], lds[slot(p, i * 4 + 2)],
+                  lds[slot(p, i * 4 + 3)]);
+            r.store(base + p * stride + i * 4);
+        }
     }
 };
 
@@ -154,12 +202,15 @@ struct RegPlane {
 // ---------------------------------------------------------------------------------------------
 // fprop / dgrad
 // ---------------------------------------------------------------------------------------------
-template <int O, int OP, typename T, int K, int H, int W>
+// GROUP: the workgroup moves the planes (GroupIO `gio`, loads already issued; `lds` is the
+// workgroup's whole LDS array), otherwise every wave its own (RegIO).
+template <int O, int OP, bool GROUP, typename T, int K, int H, int W>
 __device__ __forceinline__ void regplane_conv_body(const T *__restrict__ src,
                                                    const float *__restrict__ wt,
                                                    const float *__restrict__ bias,
-                                                   T *__restrict__ dst, float *wl, int c, int C,
-                                                   int n0, int N) {
+                                                   T *__restrict__ dst, float *lds, float *wl,
+                                                   GroupIO<T, H, W> &gio, int c, int C, int n0,
+                                                   int N) {
     constexpr bool ROW = reg_lane_is_row(O);
     using P = RegPlane<ROW, H, W>;
     using IO = RegIO<T, H, W>;
@@ -168,8 +219,10 @@ __device__ __forceinline__ void regplane_conv_body(const T *__restrict__ src,
     const unsigned lane = threadIdx.x & 63, i = lane & 15, ps = lane >> 4;
     const size_t off = ((size_t)n0 * C + c) * (H * W), stride = (size_t)C * (H * W);
     const int nvalid = N - n0;  // planes of this wave that exist (may exceed four)
+    // first plane of the workgroup's first channel (c is the channel of wave c % 8)
+    const size_t goff = off - (size_t)(c % kRegWavesPerGroup) * (H * W);
     IO io;
-    io.fetch(src + off, stride, nvalid);
+    if constexpr (!GROUP) io.fetch(src + off, stride, nvalid);
 
     // weights with duplicates folded into their representative tap (dgrad: reversed, the
     // offsets are odd-symmetric)
@@ -181,9 +234,12 @@ __device__ __forceinline__ void regplane_conv_body(const T *__restrict__ src,
         if constexpr (r >= 0 && r != s) w[r] += w[s];
     });
     const float bv = (OP == OP_FPROP && bias != nullptr) ? bias[c] : 0.f;
-    io.put(wl, nvalid);
+    if constexpr (GROUP) gio.put(lds, nvalid);
+    else io.put(wl, nvalid);
     P x;
     x.load(wl, ps, i, (int)ps < nvalid);
+    // (group mode: results go back into the wave's region once every wave has read its planes
+    // -- a chunk of the run may straddle two channels, but only in global memory, not in LDS)
     // Shift by shift: the plane shifted by SH lanes (one DPP move per register), then every
     // multiply-add whose tap has that shift.  The empty asm at the end of a shift pins the
     // running sums there, so the shifted copies die with their shift (left to itself the
@@ -211,33 +267,60 @@ __device__ __forceinline__ void regplane_conv_body(const T *__restrict__ src,
         }
     });
     y.store(wl, ps, i, (int)ps < nvalid);
-    IO::write_out(wl, dst + off, stride, nvalid);
+    if constexpr (GROUP) GroupIO<T, H, W>::write_out(lds, dst + goff, stride, nvalid);
+    else IO::write_out(wl, dst + off, stride, nvalid);
 }
 
-// any angle: every output gathers its taps from global memory through the caches (rare: the
-// networks only use the canonical orientations)
-template <int OP, typename T, int K, int H, int W>
+// any angle: same plane movement; lane i of row ps gathers row i of plane ps from the wave's
+// LDS region with the taps of the device table (rare: the networks only use the canonical
+// orientations)
+template <int OP, bool GROUP, typename T, int K, int H, int W>
 __device__ __forceinline__ void regplane_conv_table(const T *__restrict__ src,
                                                     const float *__restrict__ wt,
                                                     const float *__restrict__ bias,
                                                     const int8_t *__restrict__ dhdw,
-                                                    T *__restrict__ dst, int c, int C, int n0, int N) {
-    const unsigned lane = threadIdx.x & 63, i = lane & 15;
-    const int n = n0 + (int)(lane >> 4);
-    if (n >= N || i >= H) return;
-    const size_t off = ((size_t)n * C + c) * (H * W);
-    const float bv = (OP == OP_FPROP && bias != nullptr) ? bias[c] : 0.f;
-    for (int q = 0; q < W; q++) {
-        float acc = bv;
-        for (int s = 0; s < K; s++) {
-            const int sgn = OP == OP_DGRAD ? -1 : 1;
-            const int h = (int)i + sgn * dhdw[((size_t)c * K + s) * 2];
-            const int ww = q + sgn * dhdw[((size_t)c * K + s) * 2 + 1];
-            if (h >= 0 && h < H && ww >= 0 && ww < W)
-                acc = __builtin_fmaf(to_float(src[off + h * W + ww]), wt[(size_t)c * K + s], acc);
-        }
-        st_out(dst + off + i * W + q, from_float<T>(acc));
+                                                    T *__restrict__ dst, float *lds, float *wl,
+                                                    GroupIO<T, H, W> &gio, int c, int C, int n0,
+                                                    int N) {
+    using IO = RegIO<T, H, W>;
+    const unsigned lane = threadIdx.x & 63, i = lane & 15, ps = lane >> 4;
+    const size_t off = ((size_t)n0 * C + c) * (H * W), stride = (size_t)C * (H * W);
+    const size_t goff = off - (size_t)(c % kRegWavesPerGroup) * (H * W);
+    const int nvalid = N - n0;
+    IO io;
+    if constexpr (GROUP) {
+        gio.put(lds, nvalid);
+    } else {
+        io.fetch(src + off, stride, nvalid);
+        io.put(wl, nvalid);
     }
+    const float bv = (OP == OP_FPROP && bias != nullptr) ? bias[c] : 0.f;
+    const bool live = (int)ps < nvalid && i < H;
+    const float *plane = wl + ps * (H * W);
+    float y[W];
+#pragma unroll
+    for (int q = 0; q < W; q++) y[q] = bv;
+    for (int s = 0; s < K; s++) {
+        const int sgn = OP == OP_DGRAD ? -1 : 1;
+        const int dh = sgn * dhdw[((size_t)c * K + s) * 2], dw = sgn * dhdw[((size_t)c * K + s) * 2 + 1];
+        const float ws = wt[(size_t)c * K + s];
+        const int h = (int)i + dh;
+        if (live && h >= 0 && h < H) {
+#pragma unroll
+            for (int q = 0; q < W; q++) {
+                const int ww = q + dw;
+                if (ww >= 0 && ww < W) y[q] = __builtin_fmaf(plane[h * W + ww], ws, y[q]);
+            }
+        }
+    }
+    // every lane of the wave has read its sources before any row is overwritten
+    __builtin_amdgcn_wave_barrier();
+    if (live) {
+#pragma unroll
+        for (int q = 0; q < W; q++) wl[ps * (H * W) + i * W + q] = y[q];
+    }
+    if constexpr (GROUP) GroupIO<T, H, W>::write_out(lds, dst + goff, stride, nvalid);
+    else IO::write_out(wl, dst + off, stride, nvalid);
 }
 
 template <int OP, typename T, int K, int H, int W>
@@ -246,14 +329,43 @@ __global__ __launch_bounds__(kRegThreads) __attribute__((amdgpu_waves_per_eu(6, 
     const void *__restrict__ blob, T *__restrict__ dst, int N, int C) {
     // (wave-uniform: the weights and the class are fetched with scalar loads)
     const int c = blockIdx.x * kRegWavesPerGroup + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    if (c >= C) return;  // whole wave; the kernel has no barriers
     __shared__ __align__(16) float lds[kRegWavesPerGroup * RegIO<T, H, W>::kWaveFloats];
     float *wl = lds + (threadIdx.x >> 6) * RegIO<T, H, W>::kWaveFloats;
     const int n0 = blockIdx.y * kRegPlanesPerWave;
+    using GIO = GroupIO<T, H, W>;
+    GIO gio;
+    if constexpr (GIO::kUse) {
+        // (uniform over the grid: with whole channel blocks no wave leaves before the barriers)
+        if (C % kRegWavesPerGroup == 0) {
+            gio.fetch(src + ((size_t)n0 * C + blockIdx.x * kRegWavesPerGroup) * (H * W),
+                      (size_t)C * (H * W), N - n0);
+            const int cls = __builtin_amdgcn_readfirstlane(taps_class(blob, C, K)[c]);
+#define DWO_CASE(O)                                                                               \
+    case O:                                                                                       \
+        regplane_conv_body<O, OP, true, T, K, H, W>(src, wt, bias, dst, lds, wl, gio, c, C, n0, N); \
+        break;
+            switch (cls) {
+                DWO_CASE(0)
+                DWO_CASE(1)
+                DWO_CASE(2)
+                DWO_CASE(3)
+                DWO_CASE(4)
+                DWO_CASE(5)
+                DWO_CASE(6)
+                DWO_CASE(7)
+                default:
+                    regplane_conv_table<OP, true, T, K, H, W>(src, wt, bias, taps_dhdw(blob), dst, lds,
+                                                              wl, gio, c, C, n0, N);
+            }
+#undef DWO_CASE
+            return;
+        }
+    }
+    if (c >= C) return;  // whole wave; this path has no workgroup barriers
     const int cls = __builtin_amdgcn_readfirstlane(taps_class(blob, C, K)[c]);
-#define DWO_CASE(O)                                                             \
-    case O:                                                                     \
-        regplane_conv_body<O, OP, T, K, H, W>(src, wt, bias, dst, wl, c, C, n0, N); \
+#define DWO_CASE(O)                                                                                \
+    case O:                                                                                        \
+        regplane_conv_body<O, OP, false, T, K, H, W>(src, wt, bias, dst, lds, wl, gio, c, C, n0, N); \
         break;
     switch (cls) {
         DWO_CASE(0)
@@ -265,7 +377,8 @@ __global__ __launch_bounds__(kRegThreads) __attribute__((amdgpu_waves_per_eu(6, 
         DWO_CASE(6)
         DWO_CASE(7)
         default:
-            regplane_conv_table<OP, T, K, H, W>(src, wt, bias, taps_dhdw(blob), dst, c, C, n0, N);
+            regplane_conv_table<OP, false, T, K, H, W>(src, wt, bias, taps_dhdw(blob), dst, lds, wl, gio,
+                                                       c, C, n0, N);
     }
 #undef DWO_CASE
 }

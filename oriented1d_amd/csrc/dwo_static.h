@@ -119,13 +119,16 @@ constexpr int table_pad() {
     return K / 2 < cmax(H, W) - 1 ? K / 2 : cmax(H, W) - 1;
 }
 
+// orientation classes with a pair form (16-bit activations)
+constexpr bool pair_class(int cls) { return cls == CLS_H || cls == CLS_V; }
+
 template <int K, int H, int W, int... Os>
 constexpr int max_plane_floats(std::integer_sequence<int, Os...>) {
     constexpr int PAD = table_pad<K, H, W>();
     int m = (H + 2 * PAD) * (W + 2 * PAD + 3);  // table-driven body
     ((m = cmax(m, Geo<Os, K, tile_L<H, W>(Os), H, W>::PLANE)), ...);
-    // (pair geometries exist for row-direction orientations only, see use_pairs)
-    ((m = cmax(m, orient_class(Os) == CLS_H ? Geo<Os, K, tile_L<H, W>(Os), H, W, true>::PLANE : 0)), ...);
+    // (pair geometries of the classes that have a pair form, see use_pairs)
+    ((m = cmax(m, pair_class(orient_class(Os)) ? Geo<Os, K, tile_L<H, W>(Os), H, W, true>::PLANE : 0)), ...);
     return m;
 }
 // (a multiple of four words: planes keep the 16-byte alignment that wide LDS writes need)
@@ -180,6 +183,8 @@ struct Stager {
     static constexpr int FP = H * W / VL;              // chunks per plane
     static constexpr int PF = (PB * FP + NT - 1) / NT; // chunks per thread
     Chunk<T, VL> pre[PF];
+    Chunk<T, VL> below[PF];  // the same columns one row further down (pair staging of the
+                             // stacked class only; unused, it costs no registers)
 
     // base = first plane of the batch; `nvalid` planes of the batch exist
     __device__ __forceinline__ void prefetch(const T *__restrict__ base, unsigned plane_stride,
@@ -189,6 +194,20 @@ struct Stager {
             const unsigned f = threadIdx.x + k * NT;
             const unsigned pl = f / FP, g = f % FP;
             if (f < PB * FP && (int)pl < nvalid) pre[k].load(base + (pl * plane_stride + g * VL));
+        }
+    }
+    // the chunks one row below the ones prefetch() fetched (zeros below the last row)
+    __device__ __forceinline__ void prefetch_below(const T *__restrict__ base,
+                                                   unsigned plane_stride, int nvalid) {
+        static_assert(VL == 1 || W % VL == 0, "rows must split into whole chunks");
+#pragma unroll
+        for (int k = 0; k < PF; k++) {
+            const unsigned f = threadIdx.x + k * NT;
+            const unsigned pl = f / FP, g = f % FP;
+            if (f < PB * FP && (int)pl < nvalid) {
+                if (g + W / VL < FP) below[k].load(base + (pl * plane_stride + g * VL + W));
+                else below[k].clear();
+            }
         }
     }
     template <class Map, int PLS>
@@ -247,6 +266,27 @@ struct Stager {
                                 (unsigned)pre[k].bits(e) | (unsigned)pre[k].bits(e + 1) << 16;
                         q[2 * Map::step(3)] = pre[k].bits(3);
                         q[2 * Map::pair_step(0) + 1] = pre[k].bits(0);
+                    } else if constexpr (EH == 1 && EW == 0 && VL == 4) {
+                        // both halves of the chunk's four words are in registers (own row and
+                        // the row below): whole words, adjacent in LDS
+                        unsigned *q32 = reinterpret_cast<unsigned *>(q);
+                        typedef unsigned u4 __attribute__((ext_vector_type(4)));
+                        u4 v;
+#pragma unroll
+                        for (int e = 0; e < 4; e++)
+                            v[e] = (unsigned)pre[k].bits(e) | (unsigned)below[k].bits(e) << 16;
+                        if constexpr (Map::kWide && PLS % 4 == 0) {
+                            *reinterpret_cast<u4 *>(__builtin_assume_aligned(q32, 16)) = v;
+                        } else {
+#pragma unroll
+                            for (int e = 0; e < 4; e++) q32[e] = v[e];
+                        }
+                        // the words above the first row hold (0, x[0][w])
+                        if (r == 0) {
+                            unsigned *up = q32 + ((int)Map::index(-1, 0) - (int)Map::index(0, 0));
+#pragma unroll
+                            for (int e = 0; e < 4; e++) up[e] = (unsigned)pre[k].bits(e) << 16;
+                        }
                     } else {
 #pragma unroll
                         for (int e = 0; e < VL; e++) {
@@ -381,9 +421,9 @@ __device__ __forceinline__ void flush_out_tile(const float *lout, T *__restrict_
     for (unsigned f = threadIdx.x; f < PB * FP; f += NT) {
         const unsigned pl = f / FP, g = f % FP;
         if ((int)pl < nvalid) {
-            const float4 v = *reinterpret_cast<const float4 *>(lout + f * 4);
+            const lds_f4 v = lds_read4(lout + f * 4);
             Vec4<T> r;
-            r.set(v.x, v.y, v.z, v.w);
+            r.set(v[0], v[1], v[2], v[3]);
             r.store(obase + (pl * pstride + g * 4));
         }
     }
@@ -480,7 +520,7 @@ struct ChannelTaps {
 // words leave a thread as whole 32-bit writes) on planes whose rows split into 4-element chunks.
 template <typename T, int O, int W>
 constexpr bool use_pairs() {
-    return sizeof(T) == 2 && orient_class(O) == CLS_H && W % 4 == 0;
+    return sizeof(T) == 2 && pair_class(orient_class(O)) && W % 4 == 0;
 }
 template <int O, int OP, typename T, int K, int H, int W>
 __device__ __forceinline__ void run_canonical(const T *__restrict__ src, const float *__restrict__ wt,
@@ -504,6 +544,12 @@ __device__ __forceinline__ void run_canonical(const T *__restrict__ src, const f
 
     const T *sbase = src + (size_t)c * (H * W);
     T *dbase = dst + (size_t)c * (H * W);
+    // pair staging of the stacked class also needs every chunk's lower neighbour
+    constexpr bool BELOW = PAIR && G::CLS == CLS_V;
+    if constexpr (BELOW) {
+        sg.a.prefetch_below(sbase + (size_t)n0 * pstride, pstride, n1 - n0);
+        if (n0 + PB < n1) sg.b.prefetch_below(sbase + (size_t)(n0 + PB) * pstride, pstride, n1 - n0 - PB);
+    }
 
     constexpr bool TILE = out_tile_class<T, G::CLS>() && use_out_tile<T, H, W>();
     float *lout = lds + out_tile_offset<K, H, W>();
@@ -524,8 +570,11 @@ __device__ __forceinline__ void run_canonical(const T *__restrict__ src, const f
                 flush_out_tile<T, H, W, PB, NT>(lout, dbase + (size_t)(nb - PB) * pstride, pstride, PB);
         }
         __syncthreads();
-        if (nb + 2 * PB < n1)
+        if (nb + 2 * PB < n1) {
             stg.prefetch(sbase + (size_t)(nb + 2 * PB) * pstride, pstride, n1 - nb - 2 * PB);
+            if constexpr (BELOW)
+                stg.prefetch_below(sbase + (size_t)(nb + 2 * PB) * pstride, pstride, n1 - nb - 2 * PB);
+        }
         T *obase = dbase + (size_t)nb * pstride;  // uniform
 #pragma unroll
         for (int iter = 0; iter < ITERS; iter++) {
@@ -617,18 +666,18 @@ __device__ __forceinline__ void run_table(const T *__restrict__ src, const float
     static_assert((H + 2 * Map::PAD) * Map::RS <= PLS, "table body staging must fit the plane stride");
     const unsigned tid = threadIdx.x;
     const unsigned pstride = (unsigned)C * (H * W);
-    // live taps of this channel as LDS offsets, with their weights (dead taps never reach the
-    // plane and are skipped); kept in LDS behind the planes
-    int *toff = reinterpret_cast<int *>(lds + PB * PLS);
-    float *twt = lds + PB * PLS + K;
+    // live taps of this channel as (LDS offset, weight) pairs (dead taps never reach the plane
+    // and are skipped); kept in LDS behind the planes, read as one 8-byte broadcast per tap
+    typedef int i2 __attribute__((ext_vector_type(2)));
+    int *tapw = reinterpret_cast<int *>(lds + PB * PLS);
     __shared__ int nlive_s;
     if (tid == 0) {
         int nl = 0;
         for (int s = 0; s < K; s++) {
             const int dh = dhdw[((size_t)c * K + s) * 2], dw = dhdw[((size_t)c * K + s) * 2 + 1];
             if (dh >= H || dh <= -H || dw >= W || dw <= -W) continue;
-            toff[nl] = (OP == OP_DGRAD ? -1 : 1) * (dh * Map::RS + dw);
-            twt[nl] = wt[(size_t)c * K + s];
+            tapw[2 * nl] = (OP == OP_DGRAD ? -1 : 1) * (dh * Map::RS + dw);
+            tapw[2 * nl + 1] = __builtin_bit_cast(int, wt[(size_t)c * K + s]);
             nl++;
         }
         nlive_s = nl;
@@ -637,6 +686,9 @@ __device__ __forceinline__ void run_table(const T *__restrict__ src, const float
     for (unsigned i = tid; i < PB * PLS; i += NT) lds[i] = 0.f;
     const T *sbase = src + (size_t)c * (H * W);
     T *dbase = dst + (size_t)c * (H * W);
+    // A thread evaluates R outputs of one column, H / R rows apart: one tap read and one address
+    // serve R multiply-adds, and consecutive lanes still read consecutive words.
+    constexpr int R = H % 4 == 0 ? 4 : (H % 2 == 0 ? 2 : 1), HR = H / R;
     auto process = [&](auto &stg, int nb) {
         const int nvalid = n1 - nb;
         __syncthreads();
@@ -646,13 +698,25 @@ __device__ __forceinline__ void run_table(const T *__restrict__ src, const float
             stg.prefetch(sbase + (size_t)(nb + 2 * PB) * pstride, pstride, nvalid - 2 * PB);
         const int nlive = nlive_s;
         T *obase = dbase + (size_t)nb * pstride;
-        for (unsigned f = tid; f < PB * H * W; f += NT) {
-            const unsigned pl = f / (H * W), g = f % (H * W);
+        for (unsigned f = tid; f < PB * HR * W; f += NT) {
+            const unsigned pl = f / (HR * W), g = f % (HR * W);
             if ((int)pl >= nvalid) break;
             const float *base = lds + pl * PLS + Map::index(g / W, g % W);
-            float acc = bv;
-            for (int s = 0; s < nlive; s++) acc = __builtin_fmaf(base[toff[s]], twt[s], acc);
-            st_out(obase + (pl * pstride + g), from_float<T>(acc));
+            float acc[R];
+#pragma unroll
+            for (int k = 0; k < R; k++) acc[k] = bv;
+            for (int s = 0; s < nlive; s++) {
+                const i2 t = *reinterpret_cast<const i2 *>(__builtin_assume_aligned(tapw + 2 * s, 8));
+                // (copies first: a bit cast applied to a vector element reads element 0)
+                const int off = t[0], wbits = t[1];
+                const float *q = base + off;
+                const float ws = __builtin_bit_cast(float, wbits);
+#pragma unroll
+                for (int k = 0; k < R; k++) acc[k] = __builtin_fmaf(q[k * (HR * Map::RS)], ws, acc[k]);
+            }
+#pragma unroll
+            for (int k = 0; k < R; k++)
+                st_out(obase + (pl * pstride + g + k * (HR * W)), from_float<T>(acc[k]));
         }
     };
     for (int nb = n0; nb < n1; nb += 2 * PB) {
@@ -851,11 +915,11 @@ __device__ __forceinline__ void run_canonical_wgrad(const T *__restrict__ x, con
                 if constexpr (G::CLS == CLS_H) {
                     // one wide read: L separate reads at a lane stride of L words conflict L ways
                     if constexpr (L == 4 && W % 4 == 0 && (H * W) % 4 == 0) {
-                        const float4 dv = *reinterpret_cast<const float4 *>(g + rb * W + j * 4);
-                        d[0] = dv.x, d[1] = dv.y, d[2] = dv.z, d[3] = dv.w;
+                        const lds_f4 dv = lds_read4(g + rb * W + j * 4);
+                        d[0] = dv[0], d[1] = dv[1], d[2] = dv[2], d[3] = dv[3];
                     } else if constexpr (L == 2 && W % 2 == 0 && (H * W) % 2 == 0) {
-                        const float2 dv = *reinterpret_cast<const float2 *>(g + rb * W + j * 2);
-                        d[0] = dv.x, d[1] = dv.y;
+                        const lds_f2 dv = lds_read2(g + rb * W + j * 2);
+                        d[0] = dv[0], d[1] = dv[1];
                     } else {
 #pragma unroll
                         for (int l = 0; l < L; l++) d[l] = g[rb * W + j * L + l];
