@@ -298,10 +298,20 @@ __global__ __launch_bounds__((NhwcTile<H, W>::NT)) void nhwc_plane_kernel(
 #undef DWO_CASE
 }
 
+// register-plane kernels (dwo_regplane.h) take fprop and dgrad of planes of at most 16 x 16 when
+// the channel count is a multiple of their eight-channel blocks
+template <typename T, int K, int H, int W>
+int launch_regplane_nhwc_conv(int op, const void *src, const float *w, const float *bias,
+                              const void *taps, void *dst, int N, int C, hipStream_t st);
+
 // C must be a multiple of kSliceCh (the caller checks).
 template <typename T, int K, int H, int W>
 int launch_nhwc_plane_conv(int op, const void *src, const float *w, const float *bias,
                            const void *taps, void *dst, int N, int C, hipStream_t st) {
+    if constexpr (reg_plane_shape<H, W>()) {
+        if (N > 0 && C % 8 == 0)
+            return launch_regplane_nhwc_conv<T, K, H, W>(op, src, w, bias, taps, dst, N, C, st);
+    }
     constexpr int NT = NhwcTile<H, W>::NT, PBI = NhwcTile<H, W>::PBI;
     const size_t lds = nhwc_plane_lds_bytes<K, H, W>();
     static int cache[kMaxDevices];
@@ -427,17 +437,17 @@ __device__ __forceinline__ void wgrad_epilogue_sub(float (&acc)[K + 1], float *l
                                                    unsigned stid, int group, SlotOf slot_of) {
     constexpr int NWS = NTS / 64;
     __syncthreads();  // staged planes are dead from here on
-#pragma unroll
-    for (int s = 0; s <= K; s++) {
-        const float t = wave_sum_dpp(acc[s]);
-        if ((threadIdx.x & 63) == 63) lds[(threadIdx.x >> 6) * (K + 1) + s] = t;
-    }
+    // every lane leaves the half-wave sum of one accumulator in its wave's row of 64 words
+    lds[threadIdx.x] = wave_reduce32(acc);
     __syncthreads();
     if (stid <= K) {
         const int slot = stid == K ? K : slot_of(stid);
         float t = 0.f;
-        if (slot >= 0)
-            for (int w = 0; w < NWS; w++) t += lds[(sub * NWS + w) * (K + 1) + slot];
+        if (slot >= 0) {
+            const unsigned l = reduce32_lane(slot);
+            for (int w = 0; w < NWS; w++)
+                t += lds[(sub * NWS + w) * 64 + l] + lds[(sub * NWS + w) * 64 + 32 + l];
+        }
         out.put(c, (int)stid, group, K, t);
     }
     wgrad_finish<K>(out, lds, (c - sub) / kSliceCh, c - sub, kSliceCh);

@@ -177,6 +177,114 @@ struct GroupIO {
     }
 };
 
+// How the planes of a workgroup (eight channels c0 .. c0+7 of images n0 .. n0+3) travel between
+// global memory and the waves' LDS regions; `nvalid` = images of the block that exist.  The
+// kernels call start() before they know their orientation, put() before a wave reads its planes
+// out of its region `wl` and finish() after it wrote its results there.
+//
+// NCHW, every wave its own four planes, no workgroup barrier.
+template <typename T, int H, int W>
+struct WavePlanes {
+    static constexpr bool kBarriers = false;
+    RegIO<T, H, W> io;
+    T *out;
+    size_t stride;
+    __device__ __forceinline__ void start(const T *__restrict__ src, T *__restrict__ dst, int c,
+                                          int C, int n0, int nvalid) {
+        const size_t off = ((size_t)n0 * C + c) * (H * W);
+        stride = (size_t)C * (H * W);
+        out = dst + off;
+        io.fetch(src + off, stride, nvalid);
+    }
+    __device__ __forceinline__ void put(float *, float *wl, int nvalid) const { io.put(wl, nvalid); }
+    __device__ __forceinline__ void finish(const float *, const float *wl, int nvalid) const {
+        RegIO<T, H, W>::write_out(wl, out, stride, nvalid);
+    }
+};
+// NCHW, the workgroup moves its images' runs of eight planes (GroupIO)
+template <typename T, int H, int W>
+struct GroupPlanes {
+    static constexpr bool kBarriers = true;
+    GroupIO<T, H, W> io;
+    T *out;
+    size_t stride;
+    __device__ __forceinline__ void start(const T *__restrict__ src, T *__restrict__ dst, int c,
+                                          int C, int n0, int nvalid) {
+        const size_t off = ((size_t)n0 * C + (c - c % kRegWavesPerGroup)) * (H * W);
+        stride = (size_t)C * (H * W);
+        out = dst + off;
+        io.fetch(src + off, stride, nvalid);
+    }
+    __device__ __forceinline__ void put(float *lds, float *, int nvalid) const { io.put(lds, nvalid); }
+    __device__ __forceinline__ void finish(const float *lds, const float *, int nvalid) const {
+        GroupIO<T, H, W>::write_out(lds, out, stride, nvalid);
+    }
+};
+// NHWC: the eight channels of a pixel are 32 (16) contiguous bytes; a thread moves the slices of
+// one or two pixels, scattering them over the eight waves' regions (consecutive lanes take
+// consecutive pixels: consecutive words of each region).
+template <typename T, int H, int W>
+struct NhwcPlanes {
+    static constexpr bool kBarriers = true;
+    static constexpr int E = H * W, kWaveFloats = kRegPlanesPerWave * E;
+    static constexpr int NCH = (kRegPlanesPerWave * E + kRegThreads - 1) / kRegThreads;
+    static_assert(kRegWavesPerGroup == 8, "a slice is two four-element chunks");
+    Vec4<T> lo[NCH], hi[NCH];
+    T *out;
+    unsigned C;
+    // element offset of the slice of chunk k of this thread, or false when there is none
+    __device__ __forceinline__ bool chunk(int k, int nvalid, unsigned &p, unsigned &px) const {
+        const unsigned t = threadIdx.x + k * kRegThreads;
+        p = t / E, px = t - p * E;
+        return t < kRegPlanesPerWave * E && (int)p < nvalid;
+    }
+    __device__ __forceinline__ void start(const T *__restrict__ src, T *__restrict__ dst, int c,
+                                          int C_, int n0, int nvalid) {
+        C = (unsigned)C_;
+        const size_t off = (size_t)n0 * E * C + (c - c % kRegWavesPerGroup);
+        out = dst + off;
+#pragma unroll
+        for (int k = 0; k < NCH; k++) {
+            unsigned p, px;
+            if (chunk(k, nvalid, p, px)) {
+                const T *a = src + off + (size_t)(p * E + px) * C;
+                lo[k].load_cached(a);
+                hi[k].load_cached(a + 4);
+            }
+        }
+    }
+    __device__ __forceinline__ void put(float *lds, float *, int nvalid) const {
+#pragma unroll
+        for (int k = 0; k < NCH; k++) {
+            unsigned p, px;
+            if (chunk(k, nvalid, p, px)) {
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    lds[e * kWaveFloats + p * E + px] = lo[k].get(e);
+                    lds[(4 + e) * kWaveFloats + p * E + px] = hi[k].get(e);
+                }
+            }
+        }
+        __syncthreads();
+    }
+    __device__ __forceinline__ void finish(const float *lds, const float *, int nvalid) const {
+        __syncthreads();
+#pragma unroll
+        for (int k = 0; k < NCH; k++) {
+            unsigned p, px;
+            if (chunk(k, nvalid, p, px)) {
+                const float *q = lds + p * E + px;
+                Vec4<T> a, b;
+                a.set(q[0], q[kWaveFloats], q[2 * kWaveFloats], q[3 * kWaveFloats]);
+                b.set(q[4 * kWaveFloats], q[5 * kWaveFloats], q[6 * kWaveFloats], q[7 * kWaveFloats]);
+                T *o = out + (size_t)(p * E + px) * C;
+                a.store_cached(o);
+                b.store_cached(o + 4);
+            }
+        }
+    }
+};
+
 // A plane in registers: lane i of 16-lane row `ps` holds row i (ROW) or column i of plane ps.
 template <bool ROW, int H, int W>
 struct RegPlane {
@@ -202,27 +310,17 @@ struct RegPlane {
 // ---------------------------------------------------------------------------------------------
 // fprop / dgrad
 // ---------------------------------------------------------------------------------------------
-// GROUP: the workgroup moves the planes (GroupIO `gio`, loads already issued; `lds` is the
-// workgroup's whole LDS array), otherwise every wave its own (RegIO).
-template <int O, int OP, bool GROUP, typename T, int K, int H, int W>
-__device__ __forceinline__ void regplane_conv_body(const T *__restrict__ src,
-                                                   const float *__restrict__ wt,
-                                                   const float *__restrict__ bias,
-                                                   T *__restrict__ dst, float *lds, float *wl,
-                                                   GroupIO<T, H, W> &gio, int c, int C, int n0,
-                                                   int N) {
+// `pio` moves the planes (see WavePlanes); `lds` is the workgroup's whole LDS array, `wl` the
+// wave's region of it.
+template <int O, int OP, class PIO, int K, int H, int W>
+__device__ __forceinline__ void regplane_conv_body(const float *__restrict__ wt,
+                                                   const float *__restrict__ bias, float *lds,
+                                                   float *wl, PIO &pio, int c, int nvalid) {
     constexpr bool ROW = reg_lane_is_row(O);
     using P = RegPlane<ROW, H, W>;
-    using IO = RegIO<T, H, W>;
     constexpr int NREG = P::NREG;
     using RP = RegPlan<O, K, H, W>;  // rep[]: duplicate and dead taps
     const unsigned lane = threadIdx.x & 63, i = lane & 15, ps = lane >> 4;
-    const size_t off = ((size_t)n0 * C + c) * (H * W), stride = (size_t)C * (H * W);
-    const int nvalid = N - n0;  // planes of this wave that exist (may exceed four)
-    // first plane of the workgroup's first channel (c is the channel of wave c % 8)
-    const size_t goff = off - (size_t)(c % kRegWavesPerGroup) * (H * W);
-    IO io;
-    if constexpr (!GROUP) io.fetch(src + off, stride, nvalid);
 
     // weights with duplicates folded into their representative tap (dgrad: reversed, the
     // offsets are odd-symmetric)
@@ -234,12 +332,10 @@ __device__ __forceinline__ void regplane_conv_body(const T *__restrict__ src,
         if constexpr (r >= 0 && r != s) w[r] += w[s];
     });
     const float bv = (OP == OP_FPROP && bias != nullptr) ? bias[c] : 0.f;
-    if constexpr (GROUP) gio.put(lds, nvalid);
-    else io.put(wl, nvalid);
+    pio.put(lds, wl, nvalid);
     P x;
     x.load(wl, ps, i, (int)ps < nvalid);
-    // (group mode: results go back into the wave's region once every wave has read its planes
-    // -- a chunk of the run may straddle two channels, but only in global memory, not in LDS)
+    // (results go back into the wave's own region, which only this wave reads before finish())
     // Shift by shift: the plane shifted by SH lanes (one DPP move per register), then every
     // multiply-add whose tap has that shift.  The empty asm at the end of a shift pins the
     // running sums there, so the shifted copies die with their shift (left to itself the
@@ -267,33 +363,19 @@ __device__ __forceinline__ void regplane_conv_body(const T *__restrict__ src,
         }
     });
     y.store(wl, ps, i, (int)ps < nvalid);
-    if constexpr (GROUP) GroupIO<T, H, W>::write_out(lds, dst + goff, stride, nvalid);
-    else IO::write_out(wl, dst + off, stride, nvalid);
+    pio.finish(lds, wl, nvalid);
 }
 
 // any angle: same plane movement; lane i of row ps gathers row i of plane ps from the wave's
 // LDS region with the taps of the device table (rare: the networks only use the canonical
 // orientations)
-template <int OP, bool GROUP, typename T, int K, int H, int W>
-__device__ __forceinline__ void regplane_conv_table(const T *__restrict__ src,
-                                                    const float *__restrict__ wt,
+template <int OP, class PIO, int K, int H, int W>
+__device__ __forceinline__ void regplane_conv_table(const float *__restrict__ wt,
                                                     const float *__restrict__ bias,
-                                                    const int8_t *__restrict__ dhdw,
-                                                    T *__restrict__ dst, float *lds, float *wl,
-                                                    GroupIO<T, H, W> &gio, int c, int C, int n0,
-                                                    int N) {
-    using IO = RegIO<T, H, W>;
+                                                    const int8_t *__restrict__ dhdw, float *lds,
+                                                    float *wl, PIO &pio, int c, int nvalid) {
     const unsigned lane = threadIdx.x & 63, i = lane & 15, ps = lane >> 4;
-    const size_t off = ((size_t)n0 * C + c) * (H * W), stride = (size_t)C * (H * W);
-    const size_t goff = off - (size_t)(c % kRegWavesPerGroup) * (H * W);
-    const int nvalid = N - n0;
-    IO io;
-    if constexpr (GROUP) {
-        gio.put(lds, nvalid);
-    } else {
-        io.fetch(src + off, stride, nvalid);
-        io.put(wl, nvalid);
-    }
+    pio.put(lds, wl, nvalid);
     const float bv = (OP == OP_FPROP && bias != nullptr) ? bias[c] : 0.f;
     const bool live = (int)ps < nvalid && i < H;
     const float *plane = wl + ps * (H * W);
@@ -319,53 +401,19 @@ __device__ __forceinline__ void regplane_conv_table(const T *__restrict__ src,
 #pragma unroll
         for (int q = 0; q < W; q++) wl[ps * (H * W) + i * W + q] = y[q];
     }
-    if constexpr (GROUP) GroupIO<T, H, W>::write_out(lds, dst + goff, stride, nvalid);
-    else IO::write_out(wl, dst + off, stride, nvalid);
+    pio.finish(lds, wl, nvalid);
 }
 
-template <int OP, typename T, int K, int H, int W>
-__global__ __launch_bounds__(kRegThreads) __attribute__((amdgpu_waves_per_eu(6, 8))) void regplane_kernel(
-    const T *__restrict__ src, const float *__restrict__ wt, const float *__restrict__ bias,
-    const void *__restrict__ blob, T *__restrict__ dst, int N, int C) {
-    // (wave-uniform: the weights and the class are fetched with scalar loads)
-    const int c = blockIdx.x * kRegWavesPerGroup + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    __shared__ __align__(16) float lds[kRegWavesPerGroup * RegIO<T, H, W>::kWaveFloats];
-    float *wl = lds + (threadIdx.x >> 6) * RegIO<T, H, W>::kWaveFloats;
-    const int n0 = blockIdx.y * kRegPlanesPerWave;
-    using GIO = GroupIO<T, H, W>;
-    GIO gio;
-    if constexpr (GIO::kUse) {
-        // (uniform over the grid: with whole channel blocks no wave leaves before the barriers)
-        if (C % kRegWavesPerGroup == 0) {
-            gio.fetch(src + ((size_t)n0 * C + blockIdx.x * kRegWavesPerGroup) * (H * W),
-                      (size_t)C * (H * W), N - n0);
-            const int cls = __builtin_amdgcn_readfirstlane(taps_class(blob, C, K)[c]);
-#define DWO_CASE(O)                                                                               \
-    case O:                                                                                       \
-        regplane_conv_body<O, OP, true, T, K, H, W>(src, wt, bias, dst, lds, wl, gio, c, C, n0, N); \
-        break;
-            switch (cls) {
-                DWO_CASE(0)
-                DWO_CASE(1)
-                DWO_CASE(2)
-                DWO_CASE(3)
-                DWO_CASE(4)
-                DWO_CASE(5)
-                DWO_CASE(6)
-                DWO_CASE(7)
-                default:
-                    regplane_conv_table<OP, true, T, K, H, W>(src, wt, bias, taps_dhdw(blob), dst, lds,
-                                                              wl, gio, c, C, n0, N);
-            }
-#undef DWO_CASE
-            return;
-        }
-    }
-    if (c >= C) return;  // whole wave; this path has no workgroup barriers
+// one wave: planes of channel c, images n0 .. ; PIO::start has been called
+template <int OP, class PIO, int K, int H, int W>
+__device__ __forceinline__ void regplane_dispatch(const float *__restrict__ wt,
+                                                  const float *__restrict__ bias,
+                                                  const void *__restrict__ blob, float *lds,
+                                                  float *wl, PIO &pio, int c, int C, int nvalid) {
     const int cls = __builtin_amdgcn_readfirstlane(taps_class(blob, C, K)[c]);
-#define DWO_CASE(O)                                                                                \
-    case O:                                                                                        \
-        regplane_conv_body<O, OP, false, T, K, H, W>(src, wt, bias, dst, lds, wl, gio, c, C, n0, N); \
+#define DWO_CASE(O)                                                                    \
+    case O:                                                                            \
+        regplane_conv_body<O, OP, PIO, K, H, W>(wt, bias, lds, wl, pio, c, nvalid); \
         break;
     switch (cls) {
         DWO_CASE(0)
@@ -377,10 +425,53 @@ __global__ __launch_bounds__(kRegThreads) __attribute__((amdgpu_waves_per_eu(6, 
         DWO_CASE(6)
         DWO_CASE(7)
         default:
-            regplane_conv_table<OP, false, T, K, H, W>(src, wt, bias, taps_dhdw(blob), dst, lds, wl, gio,
-                                                       c, C, n0, N);
+            regplane_conv_table<OP, PIO, K, H, W>(wt, bias, taps_dhdw(blob), lds, wl, pio, c, nvalid);
     }
 #undef DWO_CASE
+}
+
+template <int OP, typename T, int K, int H, int W>
+__global__ __launch_bounds__(kRegThreads) __attribute__((amdgpu_waves_per_eu(6, 8))) void regplane_kernel(
+    const T *__restrict__ src, const float *__restrict__ wt, const float *__restrict__ bias,
+    const void *__restrict__ blob, T *__restrict__ dst, int N, int C) {
+    // (wave-uniform: the weights and the class are fetched with scalar loads)
+    const int c = blockIdx.x * kRegWavesPerGroup + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    __shared__ __align__(16) float lds[kRegWavesPerGroup * RegIO<T, H, W>::kWaveFloats];
+    float *wl = lds + (threadIdx.x >> 6) * RegIO<T, H, W>::kWaveFloats;
+    const int n0 = blockIdx.y * kRegPlanesPerWave;
+    if constexpr (GroupIO<T, H, W>::kUse) {
+        // (uniform over the grid: with whole channel blocks no wave leaves before the barriers)
+        if (C % kRegWavesPerGroup == 0) {
+            GroupPlanes<T, H, W> pio;
+            pio.start(src, dst, c, C, n0, N - n0);
+            regplane_dispatch<OP, GroupPlanes<T, H, W>, K, H, W>(wt, bias, blob, lds, wl, pio, c, C,
+                                                                 N - n0);
+            return;
+        }
+    }
+    if (c >= C) return;  // whole wave; this path has no workgroup barriers
+    WavePlanes<T, H, W> pio;
+    pio.start(src, dst, c, C, n0, N - n0);
+    regplane_dispatch<OP, WavePlanes<T, H, W>, K, H, W>(wt, bias, blob, lds, wl, pio, c, C, N - n0);
+}
+
+// NHWC tensors, C a multiple of eight
+template <int OP, typename T, int K, int H, int W>
+__global__ __launch_bounds__(kRegThreads) __attribute__((amdgpu_waves_per_eu(6, 8))) void regplane_nhwc_kernel(
+    const T *__restrict__ src, const float *__restrict__ wt, const float *__restrict__ bias,
+    const void *__restrict__ blob, T *__restrict__ dst, int N, int C) {
+    // Consecutive workgroup ids go to the eight XCDs in turn.  The channel blocks that share a
+    // 128-byte line of a pixel (four of fp32, eight of 16-bit types) should meet in one L2:
+    // XCD x takes the x-th eighth of the channel blocks.
+    int cb = blockIdx.x;
+    if (gridDim.x % 8 == 0) cb = (cb % 8) * (gridDim.x / 8) + cb / 8;
+    const int c = cb * kRegWavesPerGroup + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    __shared__ __align__(16) float lds[kRegWavesPerGroup * RegIO<T, H, W>::kWaveFloats];
+    float *wl = lds + (threadIdx.x >> 6) * RegIO<T, H, W>::kWaveFloats;
+    const int n0 = blockIdx.y * kRegPlanesPerWave;
+    NhwcPlanes<T, H, W> pio;
+    pio.start(src, dst, c, C, n0, N - n0);
+    regplane_dispatch<OP, NhwcPlanes<T, H, W>, K, H, W>(wt, bias, blob, lds, wl, pio, c, C, N - n0);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -400,6 +491,24 @@ int launch_regplane_conv(int op, const void *src, const float *w, const float *b
     else
         regplane_kernel<OP_DGRAD, T, K, H, W><<<grid, block, 0, st>>>((const T *)src, w, bias, taps,
                                                                      (T *)dst, N, C);
+    const hipError_t e = hipGetLastError();
+    return e == hipSuccess ? 0 : (int)e;
+}
+
+// NHWC; the caller has checked that C is a multiple of kRegWavesPerGroup
+template <typename T, int K, int H, int W>
+int launch_regplane_nhwc_conv(int op, const void *src, const float *w, const float *bias,
+                              const void *taps, void *dst, int N, int C, hipStream_t st) {
+    if (N == 0) return 0;
+    const dim3 grid(C / kRegWavesPerGroup, (N + kRegPlanesPerWave - 1) / kRegPlanesPerWave),
+        block(kRegThreads);
+    if (grid.y > 65535) return DWO_ERR_BAD_SHAPE;
+    if (op == OP_FPROP)
+        regplane_nhwc_kernel<OP_FPROP, T, K, H, W><<<grid, block, 0, st>>>((const T *)src, w, bias, taps,
+                                                                          (T *)dst, N, C);
+    else
+        regplane_nhwc_kernel<OP_DGRAD, T, K, H, W><<<grid, block, 0, st>>>((const T *)src, w, bias, taps,
+                                                                          (T *)dst, N, C);
     const hipError_t e = hipGetLastError();
     return e == hipSuccess ? 0 : (int)e;
 }

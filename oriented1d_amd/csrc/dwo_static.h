@@ -18,6 +18,12 @@
 #ifndef DWO_WGRAD_DEPTH
 #define DWO_WGRAD_DEPTH 1
 #endif
+// the same for planes of at most 16 x 16, whose register sets are one chunk per thread
+// (measured at batch 64: depth 1 / 2 / 4 = 18.8 / 21.0 / 30.8 us at 14 x 14, 11.8 / 11.5 / 11.3 us
+// at 7 x 7: these launches are not waiting for HBM)
+#ifndef DWO_WGRAD_DEPTH_SMALL
+#define DWO_WGRAD_DEPTH_SMALL 1
+#endif
 
 #include "dwo_common.h"
 #include "dwo_dispatch.h"
@@ -743,6 +749,55 @@ __device__ __forceinline__ float wave_sum_dpp(float v) {
     return v;
 }
 
+// Half-wave sums of up to 32 per-lane values, all at once.  A stage pairs every lane with a
+// partner; of two values a lane keeps one and hands the other to its partner, which kept that
+// one, so the number of values halves while the number of lanes summed doubles.  After five
+// stages (partners 7-i within eight lanes, then i^1, i^2, i^8, i^16) a lane holds the sum over
+// the 32 lanes of its half wave of value number reduce32_index(lane): about 100 vector
+// instructions for 32 values, where 32 separate wave sums take about 200 and 32 single-lane
+// stores.
+template <int CTRL>
+__device__ __forceinline__ float lane_exchange(float v) {
+    if constexpr (CTRL == 0x401F) {  // ds_swizzle, bit-mask mode (and 0x1f, or 0, xor 0x10): lane ^ 16
+        return __builtin_bit_cast(float,
+                                  __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, v), 0x401F));
+    } else {
+        return __builtin_bit_cast(
+            float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
+    }
+}
+template <int CTRL, int N>
+__device__ __forceinline__ void reduce_stage(const float (&in)[2 * N], float (&out)[N], bool sel) {
+#pragma unroll
+    for (int m = 0; m < N; m++) {
+        const float keep = sel ? in[2 * m + 1] : in[2 * m];
+        const float send = sel ? in[2 * m] : in[2 * m + 1];
+        out[m] = keep + lane_exchange<CTRL>(send);
+    }
+}
+// number of the value whose half-wave sum wave_reduce32 leaves in `lane`, and the lane (of the
+// first half wave) that holds value number idx
+__device__ __forceinline__ unsigned reduce32_index(unsigned lane) {
+    return ((lane >> 2) & 1) | (lane & 1) << 1 | ((lane >> 1) & 1) << 2 | (lane & 0x18);
+}
+__device__ __forceinline__ unsigned reduce32_lane(unsigned idx) {
+    return ((idx >> 1) & 1) | ((idx >> 2) & 1) << 1 | (idx & 1) << 2 | (idx & 0x18);
+}
+template <int NV>
+__device__ __forceinline__ float wave_reduce32(const float (&a)[NV]) {
+    static_assert(NV <= 32, "at most 32 values");
+    const unsigned lane = threadIdx.x & 63;
+    float r32[32], r16[16], r8[8], r4[4], r2[2], r1[1];
+#pragma unroll
+    for (int s = 0; s < 32; s++) r32[s] = s < NV ? a[s] : 0.f;
+    reduce_stage<0x141, 16>(r32, r16, (lane & 4) != 0);  // row_half_mirror
+    reduce_stage<0x0B1, 8>(r16, r8, (lane & 1) != 0);    // quad_perm [1,0,3,2]
+    reduce_stage<0x04E, 4>(r8, r4, (lane & 2) != 0);     // quad_perm [2,3,0,1]
+    reduce_stage<0x128, 2>(r4, r2, (lane & 8) != 0);     // row_ror:8
+    reduce_stage<0x401F, 1>(r2, r1, (lane & 16) != 0);   // lane ^ 16
+    return r1[0];
+}
+
 // Workgroup epilogue: per-thread accumulators acc[0..NV) -> wave totals (DPP) -> LDS -> one
 // value per tap handed to WgradOut.  `slot_of(s)` maps tap s to the
 // accumulator that holds its sum (-1: the tap never reaches the plane, its gradient is zero).
@@ -817,17 +872,16 @@ __device__ __forceinline__ void wgrad_epilogue(float (&acc)[K + 1], float *lds, 
                                                int c, int group, SlotOf slot_of) {
     constexpr int NW = NT / 64;
     __syncthreads();  // staged planes are dead from here on
-#pragma unroll
-    for (int s = 0; s <= K; s++) {
-        const float t = wave_sum_dpp(acc[s]);
-        if ((threadIdx.x & 63) == 63) lds[(threadIdx.x >> 6) * (K + 1) + s] = t;
-    }
+    // every lane leaves the half-wave sum of one accumulator in its wave's row of 64 words
+    lds[threadIdx.x] = wave_reduce32(acc);
     __syncthreads();
     if (threadIdx.x <= K) {
         const int slot = threadIdx.x == K ? K : slot_of(threadIdx.x);
         float t = 0.f;
-        if (slot >= 0)
-            for (int w = 0; w < NW; w++) t += lds[w * (K + 1) + slot];
+        if (slot >= 0) {
+            const unsigned l = reduce32_lane(slot);
+            for (int w = 0; w < NW; w++) t += lds[w * 64 + l] + lds[w * 64 + 32 + l];
+        }
         out.put(c, threadIdx.x, group, K, t);
     }
     wgrad_finish<K>(out, lds, c, c, 1);
@@ -884,8 +938,8 @@ __device__ __forceinline__ void run_canonical_wgrad(const T *__restrict__ x, con
 #pragma unroll
     for (int s = 0; s <= K; s++) acc[s] = 0.f;
 
-    // Two register sets per tensor keep two batches in flight while a third is being summed.
-    constexpr int DEPTH = DWO_WGRAD_DEPTH;
+    // DEPTH register sets per tensor keep that many batches in flight while another is summed.
+    constexpr int DEPTH = H * W <= 256 ? DWO_WGRAD_DEPTH_SMALL : DWO_WGRAD_DEPTH;
     Stager<T, H, W, PB, NT> sx[DEPTH], sg[DEPTH];
 #pragma unroll
     for (int k = 0; k < DEPTH; k++)
@@ -952,9 +1006,9 @@ __device__ __forceinline__ void run_canonical_wgrad(const T *__restrict__ x, con
         }
     };
     for (int nb = n0; nb < n1; nb += DEPTH * PB) {
-        process(sx[0], sg[0], nb);
-        if constexpr (DEPTH > 1)
-            if (nb + PB < n1) process(sx[DEPTH - 1], sg[DEPTH - 1], nb + PB);
+        static_for<DEPTH>([&](auto k) {
+            if (nb + k * PB < n1) process(sx[k], sg[k], nb + k * PB);
+        });
     }
     wgrad_epilogue<K, NT>(acc, lds, out, c, group, [](int s) { return (int)G::plan.rep[s]; });
 }
