@@ -413,12 +413,15 @@ template <typename T, int H, int W>
 constexpr bool use_out_tile() {
     return (H * W) % 4 == 0;
 }
-// Which classes go through the out-tile: for 16-bit activations both (2-byte stores run far
-// below the rate of wider ones); for fp32 the diagonal class only (its row-shifted 4-byte
-// stores measured 10 % slower than the tile's 16-byte ones, the stacked class's did not).
-template <typename T, int CLS>
+// Which classes go through the out-tile.  16-bit activations: the stacked and the diagonal class
+// (2-byte stores run far below the rate of wider ones).  fp32: the diagonal class (its
+// row-shifted 4-byte stores measured 10 % slower than the tile's 16-byte ones) and, on planes
+// staged one per batch, the stacked class (96 x 56 x 56, all channels at 90 degrees: fprop 42.1 ->
+// 35.1 us, dgrad 39.3 -> 37.5; at 28 x 28 it measured 3-5 % slower).  The row-direction class
+// stores 16 bytes per lane from registers and measured 5-10 % slower through the tile.
+template <typename T, int CLS, int H, int W>
 constexpr bool out_tile_class() {
-    return CLS == CLS_D || (CLS == CLS_V && sizeof(T) < 4);
+    return CLS == CLS_D || (CLS == CLS_V && (sizeof(T) < 4 || Tile<H, W>::PB == 1));
 }
 template <typename T, int H, int W, int PB, int NT>
 __device__ __forceinline__ void flush_out_tile(const float *lout, T *__restrict__ obase,
@@ -557,9 +560,49 @@ __device__ __forceinline__ void run_canonical(const T *__restrict__ src, const f
         if (n0 + PB < n1) sg.b.prefetch_below(sbase + (size_t)(n0 + PB) * pstride, pstride, n1 - n0 - PB);
     }
 
-    constexpr bool TILE = out_tile_class<T, G::CLS>() && use_out_tile<T, H, W>();
+    constexpr bool TILE = out_tile_class<T, G::CLS, H, W>() && use_out_tile<T, H, W>();
     float *lout = lds + out_tile_offset<K, H, W>();
 
+    // results of item (pl, rb, j) of the batch that starts at obase -> global memory or out-tile
+    auto emit = [&](T *obase, unsigned pl, unsigned rb, unsigned j, const float (&acc)[L]) {
+        if constexpr (G::CLS == CLS_H) {
+            T *o = obase + (pl * pstride + rb * W + j * L);
+            if constexpr (L % 4 == 0) {
+#pragma unroll
+                for (int l = 0; l < L; l += 4) {
+                    Vec4<T> r;
+                    r.set(acc[l], acc[l + 1], acc[l + 2], acc[l + 3]);
+                    r.store(o + l);
+                }
+            } else {
+#pragma unroll
+                for (int l = 0; l < L; l++) st_out(o + l, from_float<T>(acc[l]));
+            }
+        } else if constexpr (G::CLS == CLS_V) {
+            // output l sits at row rb*L + l, column j
+#pragma unroll
+            for (int l = 0; l < L; l++)
+                if (H % L == 0 || rb * L + l < H) {
+                    if constexpr (TILE)
+                        lout[pl * (H * W) + rb * (L * W) + j + l * W] = acc[l];
+                    else
+                        st_out(obase + (pl * pstride + rb * (L * W) + j) + l * W, from_float<T>(acc[l]));
+                }
+        } else {
+            // output l sits at row rb*L + P0 + l*EH, column j - Q0 + l
+#pragma unroll
+            for (int l = 0; l < L; l++) {
+                const unsigned q = j + (unsigned)(l - G::Q0);  // wraps when negative
+                const int doff = (G::P0 + l * G::EH) * W + l - G::Q0;
+                if (q < W && (H % L == 0 || rb * L + G::P0 + l * G::EH < H)) {
+                    if constexpr (TILE)
+                        lout[(int)(pl * (H * W) + rb * (L * W) + j) + doff] = acc[l];
+                    else
+                        st_out(obase + (pl * pstride + rb * (L * W) + j) + doff, from_float<T>(acc[l]));
+                }
+            }
+        }
+    };
     // Two register sets keep two batches in flight from HBM while a third is being computed.
     auto process = [&](auto &stg, int nb) {
         const int nvalid = n1 - nb;
@@ -591,45 +634,7 @@ __device__ __forceinline__ void run_canonical(const T *__restrict__ src, const f
                 const float *base = lds + (pl * PLS + rb * (G::LR * G::RS) + j);
                 float acc[L];
                 taps.accumulate(base, acc);
-                if constexpr (G::CLS == CLS_H) {
-                    T *o = obase + (pl * pstride + rb * W + j * L);
-                    if constexpr (L % 4 == 0) {
-#pragma unroll
-                        for (int l = 0; l < L; l += 4) {
-                            Vec4<T> r;
-                            r.set(acc[l], acc[l + 1], acc[l + 2], acc[l + 3]);
-                            r.store(o + l);
-                        }
-                    } else {
-#pragma unroll
-                        for (int l = 0; l < L; l++) st_out(o + l, from_float<T>(acc[l]));
-                    }
-                } else if constexpr (G::CLS == CLS_V) {
-                    // output l sits at row rb*L + l, column j
-#pragma unroll
-                    for (int l = 0; l < L; l++)
-                        if (H % L == 0 || rb * L + l < H) {
-                            if constexpr (TILE)
-                                lout[pl * (H * W) + rb * (L * W) + j + l * W] = acc[l];
-                            else
-                                st_out(obase + (pl * pstride + rb * (L * W) + j) + l * W,
-                                       from_float<T>(acc[l]));
-                        }
-                } else {
-                    // output l sits at row rb*L + P0 + l*EH, column j - Q0 + l
-#pragma unroll
-                    for (int l = 0; l < L; l++) {
-                        const unsigned q = j + (unsigned)(l - G::Q0);  // wraps when negative
-                        const int doff = (G::P0 + l * G::EH) * W + l - G::Q0;
-                        if (q < W && (H % L == 0 || rb * L + G::P0 + l * G::EH < H)) {
-                            if constexpr (TILE)
-                                lout[(int)(pl * (H * W) + rb * (L * W) + j) + doff] = acc[l];
-                            else
-                                st_out(obase + (pl * pstride + rb * (L * W) + j) + doff,
-                                       from_float<T>(acc[l]));
-                        }
-                    }
-                }
+                emit(obase, pl, rb, j, acc);
             }
         }
     };
