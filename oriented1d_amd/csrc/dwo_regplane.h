@@ -24,6 +24,12 @@
 
 namespace dwo {
 
+// Register budget of the NHWC whole-line kernel: its weights differ from row to row of a wave
+// and sit in vector registers, which does not fit the 80 registers of six waves per SIMD
+// (measured at 384 x 14 x 14 fp32: 21 us with spills at six, 15.0 at five, 13.7 at four).
+#ifndef DWO_LINE_WPE
+#define DWO_LINE_WPE 4
+#endif
 constexpr int kRegPlanesPerWave = 4;   // one per 16-lane DPP row
 constexpr int kRegWavesPerGroup = 8;   // consecutive channels per workgroup
 constexpr int kRegThreads = 64 * kRegWavesPerGroup;
@@ -186,6 +192,7 @@ struct GroupIO {
 template <typename T, int H, int W>
 struct WavePlanes {
     static constexpr bool kBarriers = false;
+    static constexpr int kPlaneStride = H * W;
     RegIO<T, H, W> io;
     T *out;
     size_t stride;
@@ -205,6 +212,7 @@ struct WavePlanes {
 template <typename T, int H, int W>
 struct GroupPlanes {
     static constexpr bool kBarriers = true;
+    static constexpr int kPlaneStride = H * W;
     GroupIO<T, H, W> io;
     T *out;
     size_t stride;
@@ -226,6 +234,7 @@ struct GroupPlanes {
 template <typename T, int H, int W>
 struct NhwcPlanes {
     static constexpr bool kBarriers = true;
+    static constexpr int kPlaneStride = H * W;
     static constexpr int E = H * W, kWaveFloats = kRegPlanesPerWave * E;
     static constexpr int NCH = (kRegPlanesPerWave * E + kRegThreads - 1) / kRegThreads;
     static_assert(kRegWavesPerGroup == 8, "a slice is two four-element chunks");
@@ -285,21 +294,101 @@ struct NhwcPlanes {
     }
 };
 
-// A plane in registers: lane i of 16-lane row `ps` holds row i (ROW) or column i of plane ps.
-template <bool ROW, int H, int W>
+// NHWC, 32 channels of one image per workgroup (C a multiple of 32): a pixel's slice is 128 (64)
+// contiguous bytes, read as 16 bytes by each of eight (four) lanes, so whole cache lines move.
+// DPP row r of wave w holds channel c0 + w + 8 r: with the networks' angle assignments
+// (round-robin over eight orientations, or eight contiguous groups) the four channels of a wave
+// share their orientation, which the straight-line bodies need.  Planes sit kPlaneStride words
+// apart, a stride that is 8 modulo 32: the 64 slices a wave scatters at a time then fall on
+// every bank twice, the minimum.
+template <typename T, int H, int W>
+struct NhwcLinePlanes {
+    static constexpr bool kBarriers = true;
+    static constexpr int E = H * W;
+    static constexpr int kPlaneStride = (E + 23) / 32 * 32 + 8;
+    static constexpr int kWaveFloats = kRegPlanesPerWave * kPlaneStride;
+    static constexpr int kBlockCh = kRegWavesPerGroup * kRegPlanesPerWave;  // 32
+    static constexpr int CPL = 16 / (int)sizeof(T);  // channels per lane: 4 or 8
+    static constexpr int LPP = kBlockCh / CPL;       // lanes per pixel: 8 or 4
+    static constexpr int NCH = (E * LPP + kRegThreads - 1) / kRegThreads;
+    static_assert(kPlaneStride >= E && kPlaneStride % 32 == 8, "plane stride");
+    Vec4<T> v[NCH][CPL / 4];
+    T *out;
+    unsigned C;
+    __device__ __forceinline__ bool chunk(int k, unsigned &px, unsigned &sub) const {
+        const unsigned t = threadIdx.x + k * kRegThreads;
+        px = t / LPP, sub = t % LPP;
+        return t < E * LPP;
+    }
+    // LDS index of channel ch (0 .. 31) of the block at pixel px
+    static __device__ __forceinline__ unsigned slot(unsigned ch, unsigned px) {
+        return (ch % kRegWavesPerGroup) * kWaveFloats + (ch / kRegWavesPerGroup) * kPlaneStride + px;
+    }
+    // c0 = first channel of the block, n = the image
+    __device__ __forceinline__ void start(const T *__restrict__ src, T *__restrict__ dst, int c0,
+                                          int C_, int n, int) {
+        C = (unsigned)C_;
+        const size_t off = (size_t)n * E * C + c0;
+        out = dst + off;
+#pragma unroll
+        for (int k = 0; k < NCH; k++) {
+            unsigned px, sub;
+            if (chunk(k, px, sub)) {
+                const T *a = src + off + (size_t)px * C + sub * CPL;
+#pragma unroll
+                for (int q = 0; q < CPL / 4; q++) v[k][q].load_cached(a + 4 * q);
+            }
+        }
+    }
+    __device__ __forceinline__ void put(float *lds, float *, int) const {
+#pragma unroll
+        for (int k = 0; k < NCH; k++) {
+            unsigned px, sub;
+            if (chunk(k, px, sub)) {
+#pragma unroll
+                for (int q = 0; q < CPL / 4; q++)
+#pragma unroll
+                    for (int e = 0; e < 4; e++) lds[slot(sub * CPL + q * 4 + e, px)] = v[k][q].get(e);
+            }
+        }
+        __syncthreads();
+    }
+    __device__ __forceinline__ void finish(const float *lds, const float *, int) const {
+        __syncthreads();
+#pragma unroll
+        for (int k = 0; k < NCH; k++) {
+            unsigned px, sub;
+            if (chunk(k, px, sub)) {
+                T *o = out + (size_t)px * C + sub * CPL;
+#pragma unroll
+                for (int q = 0; q < CPL / 4; q++) {
+                    const unsigned ch = sub * CPL + q * 4;
+                    Vec4<T> r;
+                    r.set(lds[slot(ch, px)], lds[slot(ch + 1, px)], lds[slot(ch + 2, px)],
+                          lds[slot(ch + 3, px)]);
+                    r.store_cached(o + 4 * q);
+                }
+            }
+        }
+    }
+};
+
+// A plane in registers: lane i of 16-lane row `ps` holds row i (ROW) or column i of plane ps;
+// PS = distance between the planes of a wave in its LDS region.
+template <bool ROW, int H, int W, int PS = H * W>
 struct RegPlane {
     static constexpr int NREG = ROW ? W : H, NLANE = ROW ? H : W;
     float v[NREG];
     // wl = the wave's LDS region; lanes beyond the plane (and the rows of missing planes) hold zeros
     __device__ __forceinline__ void load(const float *wl, unsigned ps, unsigned i, bool plane_ok) {
         const bool live = plane_ok && i < NLANE;
-        const float *p = wl + ps * (H * W) + (ROW ? i * W : i);
+        const float *p = wl + ps * PS + (ROW ? i * W : i);
 #pragma unroll
         for (int q = 0; q < NREG; q++) v[q] = live ? p[ROW ? q : q * W] : 0.f;
     }
     __device__ __forceinline__ void store(float *wl, unsigned ps, unsigned i, bool plane_ok) const {
         const bool live = plane_ok && i < NLANE;
-        float *p = wl + ps * (H * W) + (ROW ? i * W : i);
+        float *p = wl + ps * PS + (ROW ? i * W : i);
         if (live) {
 #pragma unroll
             for (int q = 0; q < NREG; q++) p[ROW ? q : q * W] = v[q];
@@ -311,13 +400,16 @@ struct RegPlane {
 // fprop / dgrad
 // ---------------------------------------------------------------------------------------------
 // `pio` moves the planes (see WavePlanes); `lds` is the workgroup's whole LDS array, `wl` the
-// wave's region of it.
+// wave's region of it.  `mine`: this lane's plane exists and has orientation O; `io`
+// (wave-uniform): this call also moves the planes (false when a wave makes several passes over
+// planes of different orientations and moves them itself).
 template <int O, int OP, class PIO, int K, int H, int W>
 __device__ __forceinline__ void regplane_conv_body(const float *__restrict__ wt,
                                                    const float *__restrict__ bias, float *lds,
-                                                   float *wl, PIO &pio, int c, int nvalid) {
+                                                   float *wl, PIO &pio, int c, int nvalid, bool mine,
+                                                   bool io) {
     constexpr bool ROW = reg_lane_is_row(O);
-    using P = RegPlane<ROW, H, W>;
+    using P = RegPlane<ROW, H, W, PIO::kPlaneStride>;
     constexpr int NREG = P::NREG;
     using RP = RegPlan<O, K, H, W>;  // rep[]: duplicate and dead taps
     const unsigned lane = threadIdx.x & 63, i = lane & 15, ps = lane >> 4;
@@ -332,9 +424,9 @@ __device__ __forceinline__ void regplane_conv_body(const float *__restrict__ wt,
         if constexpr (r >= 0 && r != s) w[r] += w[s];
     });
     const float bv = (OP == OP_FPROP && bias != nullptr) ? bias[c] : 0.f;
-    pio.put(lds, wl, nvalid);
+    if (io) pio.put(lds, wl, nvalid);
     P x;
-    x.load(wl, ps, i, (int)ps < nvalid);
+    x.load(wl, ps, i, mine);
     // (results go back into the wave's own region, which only this wave reads before finish())
     // Shift by shift: the plane shifted by SH lanes (one DPP move per register), then every
     // multiply-add whose tap has that shift.  The empty asm at the end of a shift pins the
@@ -362,8 +454,8 @@ __device__ __forceinline__ void regplane_conv_body(const float *__restrict__ wt,
             for (int q = 0; q < NREG; q++) asm volatile("" : "+v"(y.v[q]));
         }
     });
-    y.store(wl, ps, i, (int)ps < nvalid);
-    pio.finish(lds, wl, nvalid);
+    y.store(wl, ps, i, mine);
+    if (io) pio.finish(lds, wl, nvalid);
 }
 
 // any angle: same plane movement; lane i of row ps gathers row i of plane ps from the wave's
@@ -373,12 +465,13 @@ template <int OP, class PIO, int K, int H, int W>
 __device__ __forceinline__ void regplane_conv_table(const float *__restrict__ wt,
                                                     const float *__restrict__ bias,
                                                     const int8_t *__restrict__ dhdw, float *lds,
-                                                    float *wl, PIO &pio, int c, int nvalid) {
+                                                    float *wl, PIO &pio, int c, int nvalid, bool mine,
+                                                    bool io) {
     const unsigned lane = threadIdx.x & 63, i = lane & 15, ps = lane >> 4;
-    pio.put(lds, wl, nvalid);
+    if (io) pio.put(lds, wl, nvalid);
     const float bv = (OP == OP_FPROP && bias != nullptr) ? bias[c] : 0.f;
-    const bool live = (int)ps < nvalid && i < H;
-    const float *plane = wl + ps * (H * W);
+    const bool live = mine && i < H;
+    const float *plane = wl + ps * PIO::kPlaneStride;
     float y[W];
 #pragma unroll
     for (int q = 0; q < W; q++) y[q] = bv;
@@ -399,21 +492,22 @@ __device__ __forceinline__ void regplane_conv_table(const float *__restrict__ wt
     __builtin_amdgcn_wave_barrier();
     if (live) {
 #pragma unroll
-        for (int q = 0; q < W; q++) wl[ps * (H * W) + i * W + q] = y[q];
+        for (int q = 0; q < W; q++) wl[ps * PIO::kPlaneStride + i * W + q] = y[q];
     }
-    pio.finish(lds, wl, nvalid);
+    if (io) pio.finish(lds, wl, nvalid);
 }
 
-// one wave: planes of channel c, images n0 .. ; PIO::start has been called
+// one wave: planes of channel c (wave-uniform, or one channel per 16-lane row), orientation
+// class cls (8 and above: table-driven body), wave-uniform; PIO::start has been called
 template <int OP, class PIO, int K, int H, int W>
 __device__ __forceinline__ void regplane_dispatch(const float *__restrict__ wt,
                                                   const float *__restrict__ bias,
                                                   const void *__restrict__ blob, float *lds,
-                                                  float *wl, PIO &pio, int c, int C, int nvalid) {
-    const int cls = __builtin_amdgcn_readfirstlane(taps_class(blob, C, K)[c]);
-#define DWO_CASE(O)                                                                    \
-    case O:                                                                            \
-        regplane_conv_body<O, OP, PIO, K, H, W>(wt, bias, lds, wl, pio, c, nvalid); \
+                                                  float *wl, PIO &pio, int c, int cls, int nvalid,
+                                                  bool mine, bool io) {
+#define DWO_CASE(O)                                                                              \
+    case O:                                                                                      \
+        regplane_conv_body<O, OP, PIO, K, H, W>(wt, bias, lds, wl, pio, c, nvalid, mine, io); \
         break;
     switch (cls) {
         DWO_CASE(0)
@@ -425,7 +519,8 @@ __device__ __forceinline__ void regplane_dispatch(const float *__restrict__ wt,
         DWO_CASE(6)
         DWO_CASE(7)
         default:
-            regplane_conv_table<OP, PIO, K, H, W>(wt, bias, taps_dhdw(blob), lds, wl, pio, c, nvalid);
+            regplane_conv_table<OP, PIO, K, H, W>(wt, bias, taps_dhdw(blob), lds, wl, pio, c, nvalid,
+                                                  mine, io);
     }
 #undef DWO_CASE
 }
@@ -444,15 +539,19 @@ __global__ __launch_bounds__(kRegThreads) __attribute__((amdgpu_waves_per_eu(6, 
         if (C % kRegWavesPerGroup == 0) {
             GroupPlanes<T, H, W> pio;
             pio.start(src, dst, c, C, n0, N - n0);
-            regplane_dispatch<OP, GroupPlanes<T, H, W>, K, H, W>(wt, bias, blob, lds, wl, pio, c, C,
-                                                                 N - n0);
+            const int cls = __builtin_amdgcn_readfirstlane(taps_class(blob, C, K)[c]);
+            regplane_dispatch<OP, GroupPlanes<T, H, W>, K, H, W>(
+                wt, bias, blob, lds, wl, pio, c, cls, N - n0,
+                (int)((threadIdx.x & 63) >> 4) < N - n0, true);
             return;
         }
     }
     if (c >= C) return;  // whole wave; this path has no workgroup barriers
     WavePlanes<T, H, W> pio;
     pio.start(src, dst, c, C, n0, N - n0);
-    regplane_dispatch<OP, WavePlanes<T, H, W>, K, H, W>(wt, bias, blob, lds, wl, pio, c, C, N - n0);
+    const int cls = __builtin_amdgcn_readfirstlane(taps_class(blob, C, K)[c]);
+    regplane_dispatch<OP, WavePlanes<T, H, W>, K, H, W>(wt, bias, blob, lds, wl, pio, c, cls, N - n0,
+                                                        (int)((threadIdx.x & 63) >> 4) < N - n0, true);
 }
 
 // NHWC tensors, C a multiple of eight
@@ -471,7 +570,48 @@ __global__ __launch_bounds__(kRegThreads) __attribute__((amdgpu_waves_per_eu(6, 
     const int n0 = blockIdx.y * kRegPlanesPerWave;
     NhwcPlanes<T, H, W> pio;
     pio.start(src, dst, c, C, n0, N - n0);
-    regplane_dispatch<OP, NhwcPlanes<T, H, W>, K, H, W>(wt, bias, blob, lds, wl, pio, c, C, N - n0);
+    const int cls = __builtin_amdgcn_readfirstlane(taps_class(blob, C, K)[c]);
+    regplane_dispatch<OP, NhwcPlanes<T, H, W>, K, H, W>(wt, bias, blob, lds, wl, pio, c, cls, N - n0,
+                                                        (int)((threadIdx.x & 63) >> 4) < N - n0, true);
+}
+
+// NHWC tensors, C a multiple of 32: workgroup = 32 channels of one image (NhwcLinePlanes)
+template <int OP, typename T, int K, int H, int W>
+__global__ __launch_bounds__(kRegThreads) __attribute__((amdgpu_waves_per_eu(DWO_LINE_WPE, 8))) void regplane_nhwc_line_kernel(
+    const T *__restrict__ src, const float *__restrict__ wt, const float *__restrict__ bias,
+    const void *__restrict__ blob, T *__restrict__ dst, int N, int C) {
+    using PIO = NhwcLinePlanes<T, H, W>;
+    __shared__ __align__(16) float lds[kRegWavesPerGroup * PIO::kWaveFloats];
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    float *wl = lds + wave * PIO::kWaveFloats;
+    const int c0 = blockIdx.x * PIO::kBlockCh;
+    const int c = c0 + wave + kRegWavesPerGroup * (int)((threadIdx.x & 63) >> 4);  // per 16-lane row
+    PIO pio;
+    pio.start(src, dst, c0, C, blockIdx.y, kRegPlanesPerWave);
+    // The straight-line bodies need one orientation per pass.  A wave whose four channels share
+    // theirs (the usual case) makes one pass that also moves the planes; otherwise it moves them
+    // itself and makes one pass per distinct class, each over the rows of that class only.
+    const int cls_row = taps_class(blob, C, K)[c];
+    const int cls0 = __builtin_amdgcn_readfirstlane(cls_row);
+    constexpr int NP = kRegPlanesPerWave;
+    if (__ballot(cls_row != cls0) == 0) {
+        regplane_dispatch<OP, PIO, K, H, W>(wt, bias, blob, lds, wl, pio, c, cls0, NP, true, true);
+        return;
+    }
+    pio.put(lds, wl, NP);
+    int seen[NP];
+#pragma unroll
+    for (int r = 0; r < NP; r++) {
+        const int cls = __builtin_amdgcn_readlane(cls_row, 16 * r);
+        seen[r] = cls;
+        bool done = false;
+#pragma unroll
+        for (int q = 0; q < r; q++) done = done || seen[q] == cls;
+        if (!done)
+            regplane_dispatch<OP, PIO, K, H, W>(wt, bias, blob, lds, wl, pio, c, cls, NP,
+                                                cls_row == cls, false);
+    }
+    pio.finish(lds, wl, NP);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -500,6 +640,17 @@ template <typename T, int K, int H, int W>
 int launch_regplane_nhwc_conv(int op, const void *src, const float *w, const float *bias,
                               const void *taps, void *dst, int N, int C, hipStream_t st) {
     if (N == 0) return 0;
+    if (C % NhwcLinePlanes<T, H, W>::kBlockCh == 0 && N <= 65535) {
+        const dim3 grid(C / NhwcLinePlanes<T, H, W>::kBlockCh, N), block(kRegThreads);
+        if (op == OP_FPROP)
+            regplane_nhwc_line_kernel<OP_FPROP, T, K, H, W><<<grid, block, 0, st>>>(
+                (const T *)src, w, bias, taps, (T *)dst, N, C);
+        else
+            regplane_nhwc_line_kernel<OP_DGRAD, T, K, H, W><<<grid, block, 0, st>>>(
+                (const T *)src, w, bias, taps, (T *)dst, N, C);
+        const hipError_t e = hipGetLastError();
+        return e == hipSuccess ? 0 : (int)e;
+    }
     const dim3 grid(C / kRegWavesPerGroup, (N + kRegPlanesPerWave - 1) / kRegPlanesPerWave),
         block(kRegThreads);
     if (grid.y > 65535) return DWO_ERR_BAD_SHAPE;
