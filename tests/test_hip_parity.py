@@ -131,6 +131,22 @@ def test_stage_shapes_mixed_angles(oracle, C, HW, dtype):
     _case(oracle, 3, C, HW, HW, 31, 1, dtype, False, grouped_theta(C, 0.5), seed=HW * 5)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("C,HW", [(64, 14), (96, 7), (72, 14), (40, 7)])
+def test_nhwc_small_planes_mixed_classes(oracle, C, HW, dtype):
+    """NHWC planes held in registers: channel counts that are multiples of 32 (a wave holds
+    channels c, c+8, c+16, c+24: whole-line workgroups) and multiples of 8 only, with angle
+    layouts under which the four channels of a wave differ in class or are not canonical at all
+    (one pass per class, the table-driven pass among them), odd batch sizes."""
+    rng = np.random.default_rng(C + HW)
+    _case(oracle, 5, C, HW, HW, 31, 1, dtype, True, grouped_theta(C), seed=C * HW)
+    theta = canonical_theta(C)
+    theta[1::3] = rng.uniform(-math.pi, 2 * math.pi, len(theta[1::3])).astype(np.float32)
+    _case(oracle, 3, C, HW, HW, 31, 1, dtype, True, theta, seed=C * HW + 1)
+    theta = canonical_theta(C)[rng.permutation(C)]
+    _case(oracle, 2, C, HW, HW, 15, 1, dtype, True, theta, seed=C * HW + 2)
+
+
 @pytest.mark.parametrize("nhwc", [False, True], ids=["nchw", "nhwc"])
 @pytest.mark.parametrize("K", [7, 13, 15, 27, 31])
 def test_kernel_sizes_grouped_theta(oracle, K, nhwc):
