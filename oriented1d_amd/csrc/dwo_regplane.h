@@ -591,27 +591,21 @@ __global__ __launch_bounds__(kRegThreads) __attribute__((amdgpu_waves_per_eu(DWO
     // The straight-line bodies need one orientation per pass.  A wave whose four channels share
     // theirs (the usual case) makes one pass that also moves the planes; otherwise it moves them
     // itself and makes one pass per distinct class, each over the rows of that class only.
+    // (One loop, not unrolled, for both cases: every pass site is a copy of all nine bodies.)
     const int cls_row = taps_class(blob, C, K)[c];
-    const int cls0 = __builtin_amdgcn_readfirstlane(cls_row);
     constexpr int NP = kRegPlanesPerWave;
-    if (__ballot(cls_row != cls0) == 0) {
-        regplane_dispatch<OP, PIO, K, H, W>(wt, bias, blob, lds, wl, pio, c, cls0, NP, true, true);
-        return;
-    }
-    pio.put(lds, wl, NP);
-    int seen[NP];
-#pragma unroll
-    for (int r = 0; r < NP; r++) {
+    const bool uniform = __ballot(cls_row != __builtin_amdgcn_readfirstlane(cls_row)) == 0;
+    if (!uniform) pio.put(lds, wl, NP);
+#pragma nounroll
+    for (int r = 0; r < (uniform ? 1 : NP); r++) {
         const int cls = __builtin_amdgcn_readlane(cls_row, 16 * r);
-        seen[r] = cls;
         bool done = false;
-#pragma unroll
-        for (int q = 0; q < r; q++) done = done || seen[q] == cls;
+        for (int q = 0; q < r; q++) done = done || __builtin_amdgcn_readlane(cls_row, 16 * q) == cls;
         if (!done)
             regplane_dispatch<OP, PIO, K, H, W>(wt, bias, blob, lds, wl, pio, c, cls, NP,
-                                                cls_row == cls, false);
+                                                uniform || cls_row == cls, uniform);
     }
-    pio.finish(lds, wl, NP);
+    if (!uniform) pio.finish(lds, wl, NP);
 }
 
 // ---------------------------------------------------------------------------------------------
