@@ -61,7 +61,9 @@ def build(verbose=False, jobs=None, only=None):
     common = [hipcc()] + [f for f in HIPCC_FLAGS if f != "-shared"] + [
         "-I" + os.path.join(ROOT, "include"), "-I" + CSRC, "-c"]
     units = [(os.path.join(CSRC, "dwo_api.hip"), os.path.join(objdir, "dwo_api.o"), [])]
-    for K, H, W in PLANE_SHAPES:
+    # longest translation units first (the register-plane extents, then the largest planes): the
+    # build ends when the last worker does
+    for K, H, W in sorted(PLANE_SHAPES, key=lambda s: (s[1] > 16, -s[0], -s[1] if s[1] > 16 else s[1])):
         for t in PLANE_TYPES:
             units.append((os.path.join(CSRC, "dwo_inst.hip"),
                           os.path.join(objdir, "dwo_inst_%s_k%d_%dx%d.o" % (t, K, H, W)),

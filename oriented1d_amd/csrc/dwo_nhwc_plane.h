@@ -299,7 +299,7 @@ __global__ __launch_bounds__((NhwcTile<H, W>::NT)) void nhwc_plane_kernel(
 }
 
 // register-plane kernels (dwo_regplane.h) take fprop and dgrad of planes of at most 16 x 16 when
-// the channel count is a multiple of their eight-channel blocks
+// the channel count is a multiple of their 32-channel blocks
 template <typename T, int K, int H, int W>
 int launch_regplane_nhwc_conv(int op, const void *src, const float *w, const float *bias,
                               const void *taps, void *dst, int N, int C, hipStream_t st);
@@ -309,7 +309,7 @@ template <typename T, int K, int H, int W>
 int launch_nhwc_plane_conv(int op, const void *src, const float *w, const float *bias,
                            const void *taps, void *dst, int N, int C, hipStream_t st) {
     if constexpr (reg_plane_shape<H, W>()) {
-        if (N > 0 && C % 8 == 0)
+        if (N > 0 && N <= 65535 && C % 32 == 0)
             return launch_regplane_nhwc_conv<T, K, H, W>(op, src, w, bias, taps, dst, N, C, st);
     }
     constexpr int NT = NhwcTile<H, W>::NT, PBI = NhwcTile<H, W>::PBI;

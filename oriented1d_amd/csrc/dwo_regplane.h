@@ -228,72 +228,6 @@ struct GroupPlanes {
         GroupIO<T, H, W>::write_out(lds, out, stride, nvalid);
     }
 };
-// NHWC: the eight channels of a pixel are 32 (16) contiguous bytes; a thread moves the slices of
-// one or two pixels, scattering them over the eight waves' regions (consecutive lanes take
-// consecutive pixels: consecutive words of each region).
-template <typename T, int H, int W>
-struct NhwcPlanes {
-    static constexpr bool kBarriers = true;
-    static constexpr int kPlaneStride = H * W;
-    static constexpr int E = H * W, kWaveFloats = kRegPlanesPerWave * E;
-    static constexpr int NCH = (kRegPlanesPerWave * E + kRegThreads - 1) / kRegThreads;
-    static_assert(kRegWavesPerGroup == 8, "a slice is two four-element chunks");
-    Vec4<T> lo[NCH], hi[NCH];
-    T *out;
-    unsigned C;
-    // element offset of the slice of chunk k of this thread, or false when there is none
-    __device__ __forceinline__ bool chunk(int k, int nvalid, unsigned &p, unsigned &px) const {
-        const unsigned t = threadIdx.x + k * kRegThreads;
-        p = t / E, px = t - p * E;
-        return t < kRegPlanesPerWave * E && (int)p < nvalid;
-    }
-    __device__ __forceinline__ void start(const T *__restrict__ src, T *__restrict__ dst, int c,
-                                          int C_, int n0, int nvalid) {
-        C = (unsigned)C_;
-        const size_t off = (size_t)n0 * E * C + (c - c % kRegWavesPerGroup);
-        out = dst + off;
-#pragma unroll
-        for (int k = 0; k < NCH; k++) {
-            unsigned p, px;
-            if (chunk(k, nvalid, p, px)) {
-                const T *a = src + off + (size_t)(p * E + px) * C;
-                lo[k].load_cached(a);
-                hi[k].load_cached(a + 4);
-            }
-        }
-    }
-    __device__ __forceinline__ void put(float *lds, float *, int nvalid) const {
-#pragma unroll
-        for (int k = 0; k < NCH; k++) {
-            unsigned p, px;
-            if (chunk(k, nvalid, p, px)) {
-#pragma unroll
-                for (int e = 0; e < 4; e++) {
-                    lds[e * kWaveFloats + p * E + px] = lo[k].get(e);
-                    lds[(4 + e) * kWaveFloats + p * E + px] = hi[k].get(e);
-                }
-            }
-        }
-        __syncthreads();
-    }
-    __device__ __forceinline__ void finish(const float *lds, const float *, int nvalid) const {
-        __syncthreads();
-#pragma unroll
-        for (int k = 0; k < NCH; k++) {
-            unsigned p, px;
-            if (chunk(k, nvalid, p, px)) {
-                const float *q = lds + p * E + px;
-                Vec4<T> a, b;
-                a.set(q[0], q[kWaveFloats], q[2 * kWaveFloats], q[3 * kWaveFloats]);
-                b.set(q[4 * kWaveFloats], q[5 * kWaveFloats], q[6 * kWaveFloats], q[7 * kWaveFloats]);
-                T *o = out + (size_t)(p * E + px) * C;
-                a.store_cached(o);
-                b.store_cached(o + 4);
-            }
-        }
-    }
-};
-
 // NHWC, 32 channels of one image per workgroup (C a multiple of 32): a pixel's slice is 128 (64)
 // contiguous bytes, read as 16 bytes by each of eight (four) lanes, so whole cache lines move.
 // DPP row r of wave w holds channel c0 + w + 8 r: with the networks' angle assignments
@@ -554,27 +488,6 @@ __global__ __launch_bounds__(kRegThreads) __attribute__((amdgpu_waves_per_eu(6, 
                                                         (int)((threadIdx.x & 63) >> 4) < N - n0, true);
 }
 
-// NHWC tensors, C a multiple of eight
-template <int OP, typename T, int K, int H, int W>
-__global__ __launch_bounds__(kRegThreads) __attribute__((amdgpu_waves_per_eu(6, 8))) void regplane_nhwc_kernel(
-    const T *__restrict__ src, const float *__restrict__ wt, const float *__restrict__ bias,
-    const void *__restrict__ blob, T *__restrict__ dst, int N, int C) {
-    // Consecutive workgroup ids go to the eight XCDs in turn.  The channel blocks that share a
-    // 128-byte line of a pixel (four of fp32, eight of 16-bit types) should meet in one L2:
-    // XCD x takes the x-th eighth of the channel blocks.
-    int cb = blockIdx.x;
-    if (gridDim.x % 8 == 0) cb = (cb % 8) * (gridDim.x / 8) + cb / 8;
-    const int c = cb * kRegWavesPerGroup + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    __shared__ __align__(16) float lds[kRegWavesPerGroup * RegIO<T, H, W>::kWaveFloats];
-    float *wl = lds + (threadIdx.x >> 6) * RegIO<T, H, W>::kWaveFloats;
-    const int n0 = blockIdx.y * kRegPlanesPerWave;
-    NhwcPlanes<T, H, W> pio;
-    pio.start(src, dst, c, C, n0, N - n0);
-    const int cls = __builtin_amdgcn_readfirstlane(taps_class(blob, C, K)[c]);
-    regplane_dispatch<OP, NhwcPlanes<T, H, W>, K, H, W>(wt, bias, blob, lds, wl, pio, c, cls, N - n0,
-                                                        (int)((threadIdx.x & 63) >> 4) < N - n0, true);
-}
-
 // NHWC tensors, C a multiple of 32: workgroup = 32 channels of one image (NhwcLinePlanes)
 template <int OP, typename T, int K, int H, int W>
 __global__ __launch_bounds__(kRegThreads) __attribute__((amdgpu_waves_per_eu(DWO_LINE_WPE, 8))) void regplane_nhwc_line_kernel(
@@ -629,31 +542,19 @@ int launch_regplane_conv(int op, const void *src, const float *w, const float *b
     return e == hipSuccess ? 0 : (int)e;
 }
 
-// NHWC; the caller has checked that C is a multiple of kRegWavesPerGroup
+// NHWC; the caller has checked that C is a multiple of NhwcLinePlanes::kBlockCh
 template <typename T, int K, int H, int W>
 int launch_regplane_nhwc_conv(int op, const void *src, const float *w, const float *bias,
                               const void *taps, void *dst, int N, int C, hipStream_t st) {
     if (N == 0) return 0;
-    if (C % NhwcLinePlanes<T, H, W>::kBlockCh == 0 && N <= 65535) {
-        const dim3 grid(C / NhwcLinePlanes<T, H, W>::kBlockCh, N), block(kRegThreads);
-        if (op == OP_FPROP)
-            regplane_nhwc_line_kernel<OP_FPROP, T, K, H, W><<<grid, block, 0, st>>>(
-                (const T *)src, w, bias, taps, (T *)dst, N, C);
-        else
-            regplane_nhwc_line_kernel<OP_DGRAD, T, K, H, W><<<grid, block, 0, st>>>(
-                (const T *)src, w, bias, taps, (T *)dst, N, C);
-        const hipError_t e = hipGetLastError();
-        return e == hipSuccess ? 0 : (int)e;
-    }
-    const dim3 grid(C / kRegWavesPerGroup, (N + kRegPlanesPerWave - 1) / kRegPlanesPerWave),
-        block(kRegThreads);
-    if (grid.y > 65535) return DWO_ERR_BAD_SHAPE;
+    if (N > 65535) return DWO_ERR_BAD_SHAPE;
+    const dim3 grid(C / NhwcLinePlanes<T, H, W>::kBlockCh, N), block(kRegThreads);
     if (op == OP_FPROP)
-        regplane_nhwc_kernel<OP_FPROP, T, K, H, W><<<grid, block, 0, st>>>((const T *)src, w, bias, taps,
-                                                                          (T *)dst, N, C);
+        regplane_nhwc_line_kernel<OP_FPROP, T, K, H, W><<<grid, block, 0, st>>>((const T *)src, w, bias,
+                                                                               taps, (T *)dst, N, C);
     else
-        regplane_nhwc_kernel<OP_DGRAD, T, K, H, W><<<grid, block, 0, st>>>((const T *)src, w, bias, taps,
-                                                                          (T *)dst, N, C);
+        regplane_nhwc_line_kernel<OP_DGRAD, T, K, H, W><<<grid, block, 0, st>>>((const T *)src, w, bias,
+                                                                               taps, (T *)dst, N, C);
     const hipError_t e = hipGetLastError();
     return e == hipSuccess ? 0 : (int)e;
 }
