@@ -324,16 +324,20 @@ def main():
             torch.cuda.empty_cache()
 
     # ------------------------------------------------------------------ shapes without planes
-    # Per-kernel times of the tile kernels (any extent, stride and layout): the two stem
-    # convolutions of the networks at batch 128 (NHWC, stride 2) and the stage shapes of a 512 x 512
-    # input at batch 8 (NCHW), bf16, the networks' contiguous-group angles.
+    # Per-kernel times of shapes outside the sweep, bf16, the networks' contiguous-group angles:
+    # on the tile kernels (any extent, stride and layout) the two stem convolutions of the networks
+    # at batch 128 (NHWC, stride 2) and the stage shapes of a 512 x 512 input at batch 8 (NCHW); on
+    # the NHWC plane kernels the second convolution of the ConvNeXt-B-1D++ blocks at batch 64
+    # (4 x dim channels: the launches of the training configuration).
     other_shapes = {}
     if not args.no_extra_sweeps and not args.only:
         for tag, (N_, C_, HW_, st_, lay_) in (
                 ("stem1 128x64x224 s2 nhwc", (128, 64, 224, 2, "nhwc")),
                 ("stem2 128x64x112 s2 nhwc", (128, 64, 112, 2, "nhwc")),
                 ("8x96x128 nchw", (8, 96, 128, 1, "nchw")), ("8x192x64 nchw", (8, 192, 64, 1, "nchw")),
-                ("8x384x32 nchw", (8, 384, 32, 1, "nchw")), ("8x768x16 nchw", (8, 768, 16, 1, "nchw"))):
+                ("8x384x32 nchw", (8, 384, 32, 1, "nchw")), ("8x768x16 nchw", (8, 768, 16, 1, "nchw")),
+                ("64x512x56 nhwc", (64, 512, 56, 1, "nhwc")), ("64x1024x28 nhwc", (64, 1024, 28, 1, "nhwc")),
+                ("64x2048x14 nhwc", (64, 2048, 14, 1, "nhwc")), ("64x4096x7 nhwc", (64, 4096, 7, 1, "nhwc"))):
             nhwc = lay_ == "nhwc"
             PQ = -(-HW_ // st_)
             g = torch.Generator(device=dev).manual_seed(1)
