@@ -3,6 +3,7 @@ static device array of the library), against dwo_wgrad with a caller-allocated s
 kernels, so the results must be equal bit for bit.  Two calls in a row on the shared array, the
 second on a smaller input; then further layouts, element types and kernel families."""
 import ctypes
+import gc
 
 import numpy as np
 import pytest
@@ -41,6 +42,9 @@ def _both(N, C, H, W, K, stride, dtype, nhwc, theta, seed, with_bias=True):
     db_a = torch.full((C,), 7.0, device="cuda") if with_bias else None
     db_b = torch.full((C,), -7.0, device="cuda") if with_bias else None
     stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    # (tensors of earlier tests that sit in reference cycles are released by the collector
+    # whenever it happens to run: not between the two readings below)
+    gc.collect()
     torch.cuda.synchronize()
     print("wgrad_static case", dims, "seed", seed, flush=True)
     before = torch.cuda.memory_allocated()
