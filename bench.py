@@ -307,7 +307,7 @@ def main():
 
     # ------------------------------------------------------------------ the other rows
     # Same sweep in the other element type / layout / angle assignment (per-kernel times only,
-    # fewer repeats): bf16 NCHW, fp32 and bf16 NHWC-native, and fp32 NCHW with the networks'
+    # same launches per timing and repeats as the main table): bf16 NCHW, fp32 and bf16 NHWC-native, and fp32 NCHW with the networks'
     # contiguous-group angles.
     others = {}
     if not args.no_extra_sweeps and not args.only:
@@ -315,7 +315,7 @@ def main():
                                ("bf16", "nhwc", "roundrobin"), ("f32", "nchw", "grouped")):
             if (dt_, lay_, th_) == (args.dtype, args.layout, args.theta):
                 continue
-            r = sweep(dt_, lay_, th_, 0, 0, max(5, args.kernel_iters // 2), 3)
+            r = sweep(dt_, lay_, th_, 0, 0, args.kernel_iters, args.kernel_repeats)
             tot_us = sum(v["us"] for v in r["detail"].values())
             others["%s/%s/%s" % (dt_, lay_, th_)] = {
                 "sum_us": round(tot_us, 1),
