@@ -274,6 +274,17 @@ constexpr int tile_L(int o) {
                                     : (orient_class(o) == CLS_V ? Tile<H, W>::LV : Tile<H, W>::LD);
 }
 
+// wgrad has no outputs to store, so its row-direction items need not be a whole number of
+// 16-byte chunks: at 56 x 56 seven outputs per item make 448 items per plane, one per thread
+// (four make 784: a second pass with a quarter of the lanes idle), and a source feeds up to
+// seven running sums instead of four.  Measured with all channels at one angle: 0 degrees
+// 46.8 -> 42.3 us; 22.5 degrees (99 sources per item instead of 62) 46.7 -> 55 us, so only the
+// horizontal orientation takes it.
+template <int H, int W>
+constexpr int wgrad_L(int o) {
+    return (H == 56 && W == 56 && o == 0) ? 7 : tile_L<H, W>(o);
+}
+
 // Planes of at most 16 x 16 are handled in registers, one plane per 16-lane DPP row
 // (dwo_regplane.h), instead of being staged in LDS.
 constexpr bool reg_plane_shape_rt(int H, int W) { return H <= 16 && W <= 16; }

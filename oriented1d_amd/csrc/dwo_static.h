@@ -133,6 +133,7 @@ constexpr int max_plane_floats(std::integer_sequence<int, Os...>) {
     constexpr int PAD = table_pad<K, H, W>();
     int m = (H + 2 * PAD) * (W + 2 * PAD + 3);  // table-driven body
     ((m = cmax(m, Geo<Os, K, tile_L<H, W>(Os), H, W>::PLANE)), ...);
+    ((m = cmax(m, Geo<Os, K, wgrad_L<H, W>(Os), H, W>::PLANE)), ...);
     // (pair geometries of the classes that have a pair form, see use_pairs)
     ((m = cmax(m, pair_class(orient_class(Os)) ? Geo<Os, K, tile_L<H, W>(Os), H, W, true>::PLANE : 0)), ...);
     return m;
@@ -224,7 +225,7 @@ struct Stager {
             const unsigned pl = f / FP, g = f % FP;
             if (f < PB * FP && (int)pl < nvalid) {
                 float *plane = lds + pl * PLS;
-                if constexpr (W % VL == 0) {
+                if constexpr (W % VL == 0 && Map::kChunked) {
                     const unsigned r = g / (W / VL), w0 = (g % (W / VL)) * VL;
                     float *q = plane + Map::index(r, w0);
                     if constexpr (VL == 4 && Map::kWide && PLS % 4 == 0) {
@@ -322,6 +323,8 @@ template <class G>
 struct GeoMap {
     // rows whose four-element chunks land on 16-byte boundaries of adjacent words
     static constexpr bool kWide = G::CLS != CLS_H && G::RS % 4 == 0 && G::PL % 4 == 0;
+    // step() below holds: a four-element chunk starts at a multiple of the interleave factor
+    static constexpr bool kChunked = G::CLS != CLS_H || G::L_ < 4 || 4 % G::L_ == 0 || G::L_ % 4 == 0;
     static __device__ __forceinline__ unsigned index(int r, int w) {
         return G::interior_row(r) + G::col(w + G::PL);
     }
@@ -658,7 +661,7 @@ struct TableMap {
     static constexpr int PAD = table_pad<K, H, W>();
     static constexpr int PL = (PAD + 3) & ~3;
     static constexpr int RS = W + PL + PAD;
-    static constexpr bool kWide = RS % 4 == 0;
+    static constexpr bool kWide = RS % 4 == 0, kChunked = true;
     static __device__ __forceinline__ unsigned index(unsigned r, unsigned w) {
         return (r + PAD) * RS + w + PL;
     }
@@ -899,7 +902,7 @@ __device__ __forceinline__ void wgrad_epilogue(float (&acc)[K + 1], float *lds, 
 // row-direction classes read their L adjacent outputs as one wide word: rows stay W apart.
 template <int W, int DRS>
 struct DyMap {
-    static constexpr bool kWide = DRS % 4 == 0;
+    static constexpr bool kWide = DRS % 4 == 0, kChunked = true;
     static __device__ __forceinline__ unsigned index(unsigned r, unsigned w) { return r * DRS + w; }
     static constexpr int step(int e) { return e; }
 };
@@ -910,7 +913,7 @@ constexpr int dy_row_stride() {
 template <int K, int H, int W, int... Os>
 constexpr int max_dy_plane(std::integer_sequence<int, Os...>) {
     int m = H * W;  // table-driven body and row-direction classes
-    ((m = cmax(m, H * dy_row_stride<Geo<Os, K, tile_L<H, W>(Os), H, W>, W>())), ...);
+    ((m = cmax(m, H * dy_row_stride<Geo<Os, K, wgrad_L<H, W>(Os), H, W>, W>())), ...);
     return (m + 3) & ~3;
 }
 template <int K, int H, int W>
@@ -926,10 +929,11 @@ template <int O, typename T, int K, int H, int W>
 __device__ __forceinline__ void run_canonical_wgrad(const T *__restrict__ x, const T *__restrict__ dy,
                                                     const WgradOut &out, float *lds, int c,
                                                     int C, int n0, int n1, int group) {
-    constexpr int L = tile_L<H, W>(O);
+    constexpr int L = wgrad_L<H, W>(O);
     constexpr int PB = Tile<H, W>::PB, NT = Tile<H, W>::NT;
     using G = Geo<O, K, L, H, W>;
     constexpr int PLS = plane_floats<K, H, W>();
+    static_assert(G::PLANE <= PLS, "wgrad geometry must fit the plane stride");
     constexpr int ITERS = (PB * G::IPP + NT - 1) / NT;
     const unsigned tid = threadIdx.x;
     const unsigned pstride = (unsigned)C * (H * W);
