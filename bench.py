@@ -6,6 +6,14 @@ wgrad at each of the four ConvNeXt-T stage shapes (batch 64, K=31, theta_c = (c 
 degrees), i.e. 12 launches of the C-ABI entry points.  Inputs are resident in HBM before the
 timed region; buffer sets rotate so consecutive steps do not re-hit the 256 MB Infinity Cache.
 
+Timing protocol.  The first 20-30 ms of any burst of launches after an idle spell run up to 25 %
+slower than what follows (the power management settles the clocks); every measurement here is
+taken in the sustained state a continuous job runs in: the step loop is preceded by untimed
+steps, every per-kernel timing by at least 40 ms of launches of that kernel, and the median of
+20 repeats of 100 back-to-back launches is reported (`us`: rotating buffers, more than twice
+the 256 MB Infinity Cache per operator; `warm_us`: one fixed buffer set).  The step time right
+after the idle spell is listed beside it (`ms_per_step_first_window`).
+
 Prints ONE JSON line: `value` is the algorithmic GB/s of the whole step (sum of the 12
 operators' algorithmic bytes / step time, eager C-ABI calls); `detail` carries GB/s and the
 HBM-roofline fraction of every (shape, op); `roofline` is the dominant kernel, i.e. the one of
@@ -41,6 +49,28 @@ def algorithmic_bytes(op, N, C, H, W, K, b, stride=1):
     return act + C * K * 4 + C * K * 2
 
 
+VALU_LANES = 256 * 4 * 16   # CUs x SIMDs x lanes: one fp32 multiply-add per lane and cycle
+PEAK_CLOCK_HZ = 2.4e9       # MI355X peak engine clock
+
+
+def issue_bound_us(op_mod, theta, C, HW, K, N, clock_hz=PEAK_CLOCK_HZ):
+    """Second bound of a launch beside the HBM one: the time its multiply-adds alone occupy
+    the vector ALUs.  Per output one multiply-add per distinct tap offset that can reach the
+    plane (taps that truncation puts on the same pixel are folded into one weight, taps with
+    |dh| >= H or |dw| >= W only ever read zeros); the chip issues VALU_LANES of them per cycle
+    (packed fp32 is switched off for this library and a depthwise stencil has nothing for the
+    matrix cores).  Priced at the peak clock, so a lower bound of the bound: the sustained
+    clock under this load is lower."""
+    import torch
+
+    dh, dw = op_mod.taps_to_numpy(op_mod.build_taps(torch.from_numpy(theta), C, K), C, K)
+    fmas = 0
+    for c in range(C):
+        live = {(int(a), int(b)) for a, b in zip(dh[c], dw[c]) if abs(a) < HW and abs(b) < HW}
+        fmas += len(live)
+    return fmas * N * HW * HW / VALU_LANES / clock_hz * 1e6
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -49,9 +79,14 @@ def main():
     ap.add_argument("--dtype", default="f32", choices=list(ELEM))
     ap.add_argument("--layout", default="nchw", choices=["nchw", "nhwc"])
     ap.add_argument("--theta", default="roundrobin", choices=["roundrobin", "grouped"])
-    ap.add_argument("--kernel-iters", type=int, default=30,
+    ap.add_argument("--precondition-ms", type=float, default=60.0,
+                    help="untimed steps run for this long before the warm-up steps, so that the "
+                         "timed steps see the clocks of a continuous job")
+    ap.add_argument("--kernel-warm-ms", type=float, default=40.0,
+                    help="untimed launches of a kernel before its per-kernel timing")
+    ap.add_argument("--kernel-iters", type=int, default=100,
                     help="back-to-back launches per (shape, op) for the per-kernel timings")
-    ap.add_argument("--kernel-repeats", type=int, default=7,
+    ap.add_argument("--kernel-repeats", type=int, default=20,
                     help="repeats of the per-kernel measurement (the median is reported)")
     ap.add_argument("--no-graph", dest="graph", action="store_false",
                     help="skip the two informational hipGraph timings of the step (`value` is "
@@ -116,12 +151,16 @@ def main():
         b = ELEM[dtype]
         nhwc = layout == "nhwc"
         g = torch.Generator(device=dev).manual_seed(0)
-        nsets = max(2, math.ceil(2 * 256e6 / (2 * BATCH * 96 * 56 * 56 * b)) + 1)
+        # buffer sets per stage: the two tensors an operator touches, times the sets it rotates
+        # through, exceed twice the Infinity Cache (5 / 8 / 15 / 28 sets for fp32)
+        nsets_of = [max(2, math.ceil(2 * 256e6 / (2 * BATCH * C * HW * HW * b)) + 1)
+                    for C, HW in STAGES]
+        nsets = nsets_of[0]
         dt_code, lay_code = {"f32": 0, "bf16": 1, "f16": 2}[dtype], int(nhwc)
-        keep, calls = [], []  # calls[set][stage][op] -> zero-argument callable
-        for _ in range(nsets):
-            per_stage = []
-            for C, HW in STAGES:
+        keep, calls = [], [[] for _ in STAGES]  # calls[stage][set][op] -> zero-argument callable
+        for si, (C, HW) in enumerate(STAGES):
+            per_stage = calls[si]
+            for _ in range(nsets_of[si]):
                 shape = (BATCH, HW, HW, C) if nhwc else (BATCH, C, HW, HW)
                 x = torch.randn(shape, device=dev, generator=g).to(tdt)
                 dy = torch.randn(shape, device=dev, generator=g).to(tdt)
@@ -143,28 +182,48 @@ def main():
                     "fprop": (lambda sh=stream_h, a=fa: lib.dwo_fprop(*a, sh)),
                     "dgrad": (lambda sh=stream_h, a=da: lib.dwo_dgrad(*a, sh)),
                     "wgrad": (lambda sh=stream_h, a=wa: lib.dwo_wgrad(*a, sh)),
+                    "out": (y, dx, dw),
                 })
-            calls.append(per_stage)
+
         def checked_pass():
-            """Every call of every buffer set once, with its status checked."""
+            """Every call of every buffer set once, with its status checked and its outputs
+            tested for non-finite values."""
             for per_stage in calls:
                 for ops in per_stage:
-                    for name, fn in ops.items():
-                        _lib.check(fn(), "dwo_" + name)
+                    for name in ("fprop", "dgrad", "wgrad"):
+                        _lib.check(ops[name](), "dwo_" + name)
             torch.cuda.synchronize()
+            for per_stage in calls:
+                for ops in per_stage:
+                    for t in ops["out"]:
+                        if not bool(torch.isfinite(t).all()):
+                            raise RuntimeError("non-finite values in an operator output")
 
         checked_pass()  # any launch error surfaces here, before anything is timed
 
         def step(i):
-            for ops in calls[i % nsets]:
+            for si in range(len(STAGES)):
+                ops = calls[si][i % nsets_of[si]]
                 ops["fprop"]()
                 ops["dgrad"]()
                 ops["wgrad"]()
 
         step_bytes = sum(algorithmic_bytes(o, BATCH, C, HW, HW, KSIZE, b)
                          for C, HW in STAGES for o in ("fprop", "dgrad", "wgrad"))
-        ms_per_step, ms_eager, ms_branches, ms_graph = None, None, None, None
-        if steps > 0:
+        ms_per_step, ms_eager, ms_branches, ms_graph, ms_first = None, None, None, None, None
+        n_pre = 0
+
+        def precondition():
+            """Untimed steps for args.precondition_ms: the clocks of a continuous job."""
+            n, t0 = 0, time.perf_counter()
+            while (time.perf_counter() - t0) * 1e3 < args.precondition_ms:
+                for _ in range(8):
+                    step(n)
+                    n += 1
+                torch.cuda.synchronize()
+            return n
+
+        def timed_steps():
             for i in range(warmup):
                 step(i)
             torch.cuda.synchronize()
@@ -172,7 +231,13 @@ def main():
             for i in range(steps):
                 step(i)
             torch.cuda.synchronize()
-            ms_eager = (time.perf_counter() - t0) * 1e3 / steps
+            return (time.perf_counter() - t0) * 1e3 / steps
+
+        if steps > 0:
+            time.sleep(0.3)  # the GPU idles: what a first call after a pause sees
+            ms_first = timed_steps()
+            n_pre = precondition()
+            ms_eager = timed_steps()
             ms_per_step = ms_eager
             if args.graph:
                 # For information (not `value`): the same 12 C-ABI calls per step, captured once
@@ -183,6 +248,7 @@ def main():
                     with torch.cuda.graph(gr, stream=stream):
                         step(i)
                     graphs.append(gr)
+                precondition()
                 for i in range(warmup):
                     graphs[i % nsets].replay()
                 torch.cuda.synchronize()
@@ -204,13 +270,15 @@ def main():
                     with torch.cuda.graph(gr, stream=stream):
                         for s_ in side:
                             s_.wait_stream(stream)
-                        for ops in calls[i % nsets]:
+                        for si in range(len(STAGES)):
+                            ops = calls[si][i % nsets_of[si]]
                             ops["fprop"]()
                             ops["dgrad"](side_h[0])
                             ops["wgrad"](side_h[1])
                         for s_ in side:
                             stream.wait_stream(s_)
                     graphs.append(gr)
+                precondition()
                 for i in range(warmup):
                     graphs[i % nsets].replay()
                 torch.cuda.synchronize()
@@ -225,20 +293,27 @@ def main():
         # per-kernel timings: HIP events on the launch stream (torch's current stream is the
         # one passed to the C ABI), median over the repeats
         def timed(name, si, fixed):
-            for i in range(3):
-                calls[0 if fixed else i % nsets][si][name]()
-            torch.cuda.synchronize()
+            fns = [ops[name] for ops in calls[si]]
+            if fixed:
+                fns = fns[:1]
+            n, t0 = 0, time.perf_counter()
+            while n < 10 or (time.perf_counter() - t0) * 1e3 < args.kernel_warm_ms:
+                for _ in range(20):
+                    fns[n % len(fns)]()
+                    n += 1
+                torch.cuda.synchronize()
             reps = []
             for _ in range(kernel_repeats):
                 e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
                 e0.record(stream)
                 for i in range(kernel_iters):
-                    calls[0 if fixed else i % nsets][si][name]()
+                    fns[i % len(fns)]()
                 e1.record(stream)
                 torch.cuda.synchronize()
                 reps.append(e0.elapsed_time(e1) * 1e3 / kernel_iters)
             return sorted(reps)[len(reps) // 2]
 
+        issue_us = [issue_bound_us(op, theta_for(C, theta), C, HW, KSIZE, BATCH) for C, HW in STAGES]
         detail = {}
         for si, (C, HW) in enumerate(STAGES):
             for name in ("fprop", "dgrad", "wgrad"):
@@ -249,11 +324,15 @@ def main():
                 ab = algorithmic_bytes(name, BATCH, C, HW, HW, KSIZE, b)
                 gbs = ab / (us * 1e-6) / 1e9
                 detail[key] = {"us": round(us, 2), "GB/s": round(gbs, 1),
-                               "frac_hbm": round(gbs / HBM_PEAK_GBS, 4), "bytes": ab}
+                               "frac_hbm": round(gbs / HBM_PEAK_GBS, 4), "bytes": ab,
+                               "hbm_bound_us": round(ab / HBM_PEAK_GBS / 1e3, 2),
+                               "issue_bound_us": round(issue_us[si], 2)}
                 if warm:
                     detail[key]["warm_us"] = round(timed(name, si, True), 2)
         copy_src = keep[0]
         res = {"ms_per_step": ms_per_step, "ms_per_step_eager": ms_eager,
+               "ms_per_step_first_window": ms_first, "precondition_steps": n_pre,
+               "nsets_per_stage": nsets_of,
                "ms_per_step_branches": ms_branches, "ms_per_step_graph": ms_graph, "detail": detail,
                "nsets": nsets,
                "step_bytes": step_bytes, "copy_src": copy_src if args.calibration_copy else None}
@@ -265,6 +344,8 @@ def main():
     main_res_eager = main_res["ms_per_step_eager"]
     main_res_graph, main_res_branches = main_res["ms_per_step_graph"], main_res["ms_per_step_branches"]
     nsets, step_bytes = main_res["nsets"], main_res["step_bytes"]
+    nsets_per_stage, ms_first = main_res["nsets_per_stage"], main_res["ms_per_step_first_window"]
+    n_pre = main_res["precondition_steps"]
     value = step_bytes / (ms_per_step * 1e-3) / 1e9
 
     if args.calibration_copy:
@@ -298,7 +379,12 @@ def main():
                     "achieved": dom["GB/s"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
                     "frac": round(dom["GB/s"] / HBM_PEAK_GBS, 4),
                     "traffic": traffic.get(dom_key),
-                    "launch_us": dom["us"], "algorithmic_bytes": dom["bytes"]}
+                    "launch_us": dom["us"], "algorithmic_bytes": dom["bytes"],
+                    "hbm_bound_us": dom["hbm_bound_us"], "issue_bound_us": dom["issue_bound_us"],
+                    "binding_bound": "hbm" if dom["hbm_bound_us"] >= dom["issue_bound_us"] else "valu issue",
+                    "issue_bound": "multiply-adds after folding duplicate and dead taps / (%d lanes "
+                                   "x %.1f GHz peak clock), no packed fp32, no matrix cores"
+                                   % (VALU_LANES, PEAK_CLOCK_HZ / 1e9)}
         low_key = min(detail, key=lambda k: detail[k]["frac_hbm"])
         roofline_min = {"kernel": low_key, "frac": detail[low_key]["frac_hbm"],
                         "launch_us": detail[low_key]["us"],
@@ -317,10 +403,17 @@ def main():
                 continue
             r = sweep(dt_, lay_, th_, 0, 0, args.kernel_iters, args.kernel_repeats)
             tot_us = sum(v["us"] for v in r["detail"].values())
+            tr_ = {}
+            tp_ = os.path.join(ROOT, "profiles", "dwoconv1d_stage_sweep_%s_%s_hbm_traffic.json"
+                               % (dt_, lay_))
+            if th_ == "roundrobin" and os.path.exists(tp_):
+                with open(tp_) as fh:
+                    tr_ = json.load(fh).get("traffic_bytes_per_launch", {})
             others["%s/%s/%s" % (dt_, lay_, th_)] = {
                 "sum_us": round(tot_us, 1),
                 "GB/s": round(r["step_bytes"] / tot_us / 1e3, 1),
-                "ops": {k: [v["us"], v["frac_hbm"]] for k, v in r["detail"].items()}}
+                "ops": {k: [v["us"], v["frac_hbm"]] for k, v in r["detail"].items()},
+                "traffic": {k: tr_.get(k) for k in r["detail"]} if tr_ else None}
             torch.cuda.empty_cache()
 
     # ------------------------------------------------------------------ shapes without planes
@@ -358,17 +451,28 @@ def main():
                              lib.dwo_wgrad(*a))}
             row = {}
             torch.cuda.synchronize()  # inputs were made on torch's stream, the calls run on `stream`
+            outs_ = {"fprop": y, "dgrad": dx, "wgrad": dw}
             for name, fn in fns.items():
                 _lib.check(fn(), "dwo_" + name)
                 torch.cuda.synchronize()
-                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-                e0.record(stream)
-                for _ in range(10):
-                    fn()
-                e1.record(stream)
-                torch.cuda.synchronize()
-                us = e0.elapsed_time(e1) * 100.0
+                t0 = time.perf_counter()
+                while (time.perf_counter() - t0) * 1e3 < args.kernel_warm_ms:
+                    for _ in range(5):
+                        fn()
+                    torch.cuda.synchronize()
+                reps = []
+                for _ in range(5):
+                    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                    e0.record(stream)
+                    for _ in range(20):
+                        fn()
+                    e1.record(stream)
+                    torch.cuda.synchronize()
+                    reps.append(e0.elapsed_time(e1) * 50.0)
+                us = sorted(reps)[2]
                 ab = algorithmic_bytes(name, N_, C_, HW_, HW_, KSIZE, 2, st_)
+                if not bool(torch.isfinite(outs_[name]).all()):
+                    raise RuntimeError("non-finite values in %s of %s" % (name, tag))
                 row[name] = [round(us, 1), round(ab / us / 1e3 / HBM_PEAK_GBS, 4)]
             other_shapes[tag] = row
             del x, dy, y, dx, scr
@@ -482,8 +586,14 @@ def main():
         imgs = torch.randn(128, 3, 224, 224, device=dev).to(torch.bfloat16)
         with torch.no_grad():
             for _ in range(2):
-                model(imgs)
+                logits = model(imgs)
             torch.cuda.synchronize()
+            if logits.shape != (128, 1000) or not bool(torch.isfinite(logits).all()):
+                raise RuntimeError("ConvNeXt-T-1D forward: wrong shape or non-finite logits")
+            w0 = time.perf_counter()  # the clocks of a continuous job before the timed forwards
+            while (time.perf_counter() - w0) * 1e3 < args.precondition_ms:
+                model(imgs)
+                torch.cuda.synchronize()
             m0 = time.perf_counter()
             for _ in range(args.model_iters):
                 model(imgs)
@@ -553,10 +663,14 @@ def main():
                     loss = torch.nn.functional.cross_entropy(net(imgs).float(), labels)
                 loss.backward()
                 opt.step()
+                return loss
 
             for _ in range(2):
-                train_step()
+                loss_ = train_step()
             torch.cuda.synchronize()
+            if not math.isfinite(float(loss_)) or not all(
+                    bool(torch.isfinite(p_).all()) for p_ in net.parameters()):
+                raise RuntimeError("ConvNeXt-B-1D++ training step: non-finite loss or parameters")
             t0 = time.perf_counter()
             for _ in range(args.train_iters):
                 train_step()
@@ -578,11 +692,16 @@ def main():
                 outs = net(imgs)
                 if not targets:
                     targets.extend(torch.randn_like(o) for o in outs)
-                sum((o.float() * r.float()).sum() for o, r in zip(outs, targets)).backward()
+                loss = sum((o.float() * r.float()).sum() for o, r in zip(outs, targets))
+                loss.backward()
+                return loss
 
             for _ in range(2):
-                feature_step()
+                loss_ = feature_step()
             torch.cuda.synchronize()
+            if not math.isfinite(float(loss_)) or not all(
+                    p_.grad is None or bool(torch.isfinite(p_.grad).all()) for p_ in net.parameters()):
+                raise RuntimeError("ConvNeXt-T-1D features step: non-finite loss or gradients")
             t0 = time.perf_counter()
             for _ in range(args.train_iters):
                 feature_step()
@@ -604,7 +723,14 @@ def main():
         "config": {"workload": "dwoconv1d fprop+dgrad+wgrad sweep at ConvNeXt-T stage shapes "
                                "(C=96@56x56, 192@28x28, 384@14x14, 768@7x7), batch 64, K=31, "
                                "8 orientations %s, stride 1" % args.theta,
-                   "layout": args.layout, "buffer_sets": nsets,
+                   "layout": args.layout, "buffer_sets_per_stage": nsets_per_stage,
+                   "timing": "sustained state: %d untimed steps (%.0f ms) run before the warm-up "
+                             "steps; the same warm-up + timed steps right after an idle spell are "
+                             "ms_per_step_first_window; per-kernel: >= %.0f ms of launches, then "
+                             "the median of %d x %d launches"
+                             % (n_pre, args.precondition_ms, args.kernel_warm_ms,
+                                args.kernel_repeats, args.kernel_iters),
+                   "ms_per_step_first_window": round(ms_first, 4) if ms_first else None,
                    "launch": "eager C-ABI calls on one stream (value, ms_per_step); the hipGraph "
                              "replays of the same step are listed for information",
                    "ms_per_step_graph": round(main_res_graph, 4) if main_res_graph else None,

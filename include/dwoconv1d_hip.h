@@ -119,11 +119,21 @@ int dwo_dgrad(const void *dy, const float *w, const void *taps, void *dx,
 /*
  * wgrad -- replaces `wgrad(dy, x, theta)` (models/dwoconv1d/kernels/kernels.cu:42-54) and,
  * when `db` is non-NULL, the bias gradient `dy.sum([0,2,3])` of dwoconv1d.py:66-67.
- * Two-stage and deterministic: workgroups write partial sums into `scratch`
- * (`dwo_wgrad_scratch_bytes` bytes, caller-allocated, contents undefined on entry and
- * exit) and one second-stage kernel reduces them in a fixed order -- no atomics, unlike
- * models/dwoconv1d/kernels/kernels.h:504-517.  dw: [C,K] fp32 (fully overwritten);
- * db: [C] fp32 or NULL.
+ * Deterministic: workgroups write partial sums into `scratch` (`dwo_wgrad_scratch_bytes`
+ * bytes, caller-allocated, contents undefined on entry and exit) and the partial sums of a
+ * channel are added in a fixed order -- no floating-point atomics, unlike
+ * models/dwoconv1d/kernels/kernels.h:504-517.  For the stride-1 plane shapes that addition
+ * happens inside the same kernel (the last workgroup of a channel to finish does it, found by
+ * an integer counter in device memory the library owns); otherwise, and always under stream
+ * capture, a second small kernel does it.  Both give the same bits.
+ * dw: [C,K] fp32 (fully overwritten); db: [C] fp32 or NULL.
+ *
+ * Concurrency.  Calls on one stream are ordered.  Calls on different streams may overlap as long
+ * as they do not share `scratch` (or `dw`/`db`): the library's counters belong to the stream
+ * (the first 64 streams that call wgrad on a device each get a set; calls on further streams,
+ * on hipStreamPerThread and under capture use the second kernel instead), so no two launches
+ * that can run at the same time count on the same counters.  A captured graph contains no
+ * reference to library-owned memory.
  */
 size_t dwo_wgrad_scratch_bytes(int N, int C, int H, int W, int K, int stride, int dtype,
                                int layout);
@@ -147,6 +157,14 @@ int dwo_wgrad(const void *dy, const void *x, const void *taps, float *dw, float 
 int dwo_wgrad_static(const void *dy, const void *x, const void *taps, float *dw, float *db,
                      int N, int C, int H, int W, int K, int stride, int dtype, int layout,
                      void *stream);
+
+/*
+ * Where the partial sums of the stride-1 plane wgrad kernels are added up: in_kernel != 0 (the
+ * default) inside the kernel that produced them, 0 in a second kernel.  The results are
+ * bit-identical; the switch exists so that both paths can be exercised and compared.  No
+ * counterpart in the reference.  Process-wide; returns the previous setting.
+ */
+int dwo_set_wgrad_reduction(int in_kernel);
 
 /*
  * fprop of a pointwise-projected NHWC tensor without materialising it: y = fprop(pw(x)) with

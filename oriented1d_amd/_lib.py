@@ -24,6 +24,7 @@ SIGNATURES = {
     "dwo_wgrad_scratch_bytes": (_sz, [_i] * 8),
     "dwo_wgrad": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _sz] + [_i] * 8 + [_vp]),
     "dwo_wgrad_static": (_i, [_vp, _vp, _vp, _vp, _vp] + [_i] * 8 + [_vp]),
+    "dwo_set_wgrad_reduction": (_i, [_i]),
     "dwo_pointwise_fprop_nhwc": (_i, [_vp] * 7 + [_i] * 8 + [_vp]),
     "dwo_layernorm_nhwc": (_i, [_vp, _vp, _vp, _vp, _sz, _i, ctypes.c_float, _i, _i, _vp]),
     "dwo_nchw_layernorm_nhwc": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, ctypes.c_float, _i, _vp]),
@@ -57,14 +58,28 @@ _ready = set()
 def ready(device):
     """The loaded library with its kernels set up on ``device`` (a torch CUDA device): the first
     use on a device runs ``dwo_init`` there, so no later call does anything but launch kernels."""
-    lib = load()
-    if device.index not in _ready:
-        import torch
+    import torch
 
-        with torch.cuda.device(device):
+    lib = load()
+    index = device.index if device.index is not None else torch.cuda.current_device()
+    if index not in _ready:
+        with torch.cuda.device(index):
             check(lib.dwo_init(), "dwo_init")
-        _ready.add(device.index)
+        _ready.add(index)
     return lib
+
+
+def launch(device, fn, *args):
+    """Calls a launching entry point with ``device`` current: the library keeps its per-device
+    state (occupancy figures, counters, the static scratch) under the current device, which
+    must be the one the tensors and the stream live on."""
+    import torch
+
+    index = device.index if device.index is not None else torch.cuda.current_device()
+    if index == torch.cuda.current_device():
+        return fn(*args)
+    with torch.cuda.device(index):
+        return fn(*args)
 
 
 def check(status, what):

@@ -7,6 +7,7 @@
 #include <string.h>
 
 #include <atomic>
+#include <mutex>
 
 #include "dwo_common.h"
 #include "dwo_generic.h"
@@ -275,33 +276,75 @@ int dgrad_t(const void *dy, const float *w, const void *taps, void *dx, const Co
     return launch_status();
 }
 
-// Ticket counters of the plane wgrad kernels (wgrad_finish): one counter per channel block and
-// launch.  They live in the library's device image, zero when the library is loaded, and every
-// launch leaves its counters at zero again.  Launches that may run at the same time must not
-// share counters, so each call takes the next of kTicketSlots rows; a row is reused
-// kTicketSlots calls later, long after the launch that used it has drained (a device runs a
-// handful of kernels at once).  Shapes with more channel blocks than a row holds, and devices
-// where the symbol cannot be resolved, take the separate reduction kernel instead.
+// Ticket counters of the plane wgrad kernels (wgrad_finish): one counter per channel block.  They
+// live in the library's device image, zero when the library is loaded (dwo_init clears them
+// again), and every launch leaves its counters at zero.  Launches that may run at the same time
+// must not share counters, so a row of counters belongs to one stream: launches on a stream run
+// one after the other, and the first kTicketSlots streams that call wgrad on a device each own a
+// row for good.  Everything else takes the separate reduction kernel (bit-identical results):
+// calls under stream capture (a graph would keep its row while eager calls go on using it, and
+// two replays of one graph may overlap), the per-thread default stream (one handle, many
+// streams), further streams once the rows are taken, shapes with more channel blocks than a row
+// holds, and devices where the symbol cannot be resolved.
 constexpr int kTicketSlots = 64, kTicketRow = 4096;
 static __device__ unsigned g_tickets[kTicketSlots * kTicketRow];
-unsigned *g_tickets_ptr[kMaxDevices];
-std::atomic<unsigned> g_ticket_next{0};
+struct TicketRows {
+    std::mutex mu;
+    unsigned *base = nullptr;
+    int used = 0;
+    hipStream_t owner[kTicketSlots];
+};
+TicketRows g_ticket_rows[kMaxDevices];
+std::atomic<int> g_tickets_enabled{1};  // dwo_set_wgrad_reduction
 
-unsigned *ticket_row(int blocks) {
-    if (blocks > kTicketRow) return nullptr;
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return nullptr;
-    unsigned *p = __atomic_load_n(&g_tickets_ptr[dev], __ATOMIC_ACQUIRE);
-    if (p == nullptr) {
+// the device's counter array (resolved once per device), or null
+unsigned *ticket_base(TicketRows &rows) {
+    if (rows.base == nullptr) {
         void *sym = nullptr;
         if (hipGetSymbolAddress(&sym, HIP_SYMBOL(g_tickets)) != hipSuccess || sym == nullptr) {
             (void)hipGetLastError();
             return nullptr;
         }
-        p = (unsigned *)sym;
-        __atomic_store_n(&g_tickets_ptr[dev], p, __ATOMIC_RELEASE);
+        rows.base = (unsigned *)sym;
     }
-    return p + (size_t)(g_ticket_next.fetch_add(1, std::memory_order_relaxed) % kTicketSlots) * kTicketRow;
+    return rows.base;
+}
+
+unsigned *ticket_row(int blocks, hipStream_t st) {
+    if (blocks > kTicketRow || !g_tickets_enabled.load(std::memory_order_relaxed)) return nullptr;
+    if (st == hipStreamPerThread) return nullptr;
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(st, &cap) != hipSuccess) {
+        (void)hipGetLastError();
+        return nullptr;
+    }
+    if (cap != hipStreamCaptureStatusNone) return nullptr;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return nullptr;
+    TicketRows &rows = g_ticket_rows[dev];
+    std::lock_guard<std::mutex> lock(rows.mu);
+    unsigned *base = ticket_base(rows);
+    if (base == nullptr) return nullptr;
+    int r = 0;
+    while (r < rows.used && rows.owner[r] != st) r++;
+    if (r == rows.used) {
+        if (rows.used == kTicketSlots) return nullptr;
+        rows.owner[rows.used++] = st;
+    }
+    return base + (size_t)r * kTicketRow;
+}
+
+// dwo_init: the counters back to zero (they already are unless a launch was torn down half way)
+int reset_tickets() {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return DWO_OK;
+    TicketRows &rows = g_ticket_rows[dev];
+    std::lock_guard<std::mutex> lock(rows.mu);
+    unsigned *base = ticket_base(rows);
+    if (base == nullptr) return DWO_OK;
+    hipError_t e = hipDeviceSynchronize();
+    if (e == hipSuccess) e = hipMemset(base, 0, sizeof(unsigned) * kTicketSlots * kTicketRow);
+    return e == hipSuccess ? DWO_OK : (int)e;
 }
 
 template <typename T>
@@ -311,11 +354,11 @@ int wgrad_t(const void *dy, const void *x, const void *taps, float *dw, float *d
     int rc, NG = 0;
     bool direct = false;  // stage 1 wrote dw / db itself (one group per channel, or tickets)
     if (plane_batch(d, layout) != 0) {
-        unsigned *tickets = ticket_row(d.C);
+        unsigned *tickets = ticket_row(d.C, st);
         rc = try_plane_wgrad<T>(x, dy, taps, part, dw, db, tickets, &NG, d, st);
         direct = NG == 1 || tickets != nullptr;
     } else if (nhwc_plane_batch(d, layout) != 0) {
-        unsigned *tickets = ticket_row(d.C / kSliceCh);
+        unsigned *tickets = ticket_row(d.C / kSliceCh, st);
         rc = try_nhwc_plane_wgrad<T>(x, dy, taps, part, dw, db, tickets, &NG, d, st);
         direct = NG == 1 || tickets != nullptr;
     } else if (tile_covers(d, layout, sizeof(T))) {
@@ -427,7 +470,8 @@ int dwo_init(void) {
     void *scratch = nullptr;  // the static wgrad scratch's address on this device
     const int rc = static_scratch(&scratch);
     if (rc != DWO_OK) return rc;
-    (void)ticket_row(1);  // and the ticket counters' (a row taken here is simply skipped)
+    const int trc = reset_tickets();  // and the ticket counters', all zero from here on
+    if (trc != DWO_OK) return trc;
     // (the set-up calls leave their own failures in the runtime's last-error slot)
     (void)init_type<float>();
     (void)init_type<bf16_t>();
@@ -435,7 +479,11 @@ int dwo_init(void) {
     return launch_status();
 }
 
-int dwo_version(void) { return 200; }
+int dwo_version(void) { return 300; }
+
+int dwo_set_wgrad_reduction(int in_kernel) {
+    return g_tickets_enabled.exchange(in_kernel ? 1 : 0, std::memory_order_relaxed);
+}
 
 const char *dwo_status_string(int status) {
     switch (status) {

@@ -531,7 +531,7 @@ int launch_regplane_conv(int op, const void *src, const float *w, const float *b
     const dim3 grid((C + kRegWavesPerGroup - 1) / kRegWavesPerGroup,
                     (N + kRegPlanesPerWave - 1) / kRegPlanesPerWave),
         block(kRegThreads);
-    if (grid.y > 65535) return DWO_ERR_BAD_SHAPE;
+    if (grid.y > 65535) return -100;  // not covered: the dispatch goes on to the tile kernels
     if (op == OP_FPROP)
         regplane_kernel<OP_FPROP, T, K, H, W><<<grid, block, 0, st>>>((const T *)src, w, bias, taps,
                                                                      (T *)dst, N, C);

@@ -42,6 +42,39 @@ __device__ __forceinline__ void static_for(F &&f) {
 
 
 
+// All of the wave's outstanding global loads and stores have completed.  The kernels call this
+// once per staged batch, unconditionally, right before the staged registers are written to LDS
+// (which has to wait for them anyway).  Stated in straight-line code it also tells the compiler
+// that nothing is pending when the next prefetch is issued: left to itself it places a full wait
+// inside every conditionally executed load and LDS write of the batch loop (a load's address
+// is computed in the registers the load will fill, which on some path still look busy), so
+// that the second load of a batch was only issued after the first had come back from HBM.
+__device__ __forceinline__ void wait_vmem_done() {
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0), expcnt and lgkmcnt untouched
+}
+
+// Issue priority of the calling wave for its next staged batch, from the share of its batches it
+// has finished: 3 at the start, falling to 0 in the last quarter.  The CU's instruction arbiter
+// serves waves of equal priority oldest first, so of the workgroups that share a CU the one
+// dispatched first ran at close to full speed and the last one crawled until the others had
+// left: at 96 x 56 x 56 the workgroups of an fprop launch ended between 17 and 35 us after its
+// start, and a CU spent the last third of the launch with one or two workgroups.  With the
+// priority tied to progress a workgroup that is ahead yields to the ones behind it, whatever the
+// dispatch order was: the same launch's workgroups end between 25.5 and 32.6 us, the launch
+// 11 % earlier.
+__device__ __forceinline__ void set_progress_priority(int done, int total) {
+    const int p = 3 - min(3, done * 4 / total);
+    if (p == 0) __builtin_amdgcn_s_setprio(0);
+    else if (p == 1) __builtin_amdgcn_s_setprio(1);
+    else if (p == 2) __builtin_amdgcn_s_setprio(2);
+    else __builtin_amdgcn_s_setprio(3);
+}
+// (planes below 10 x 10: the eight-plane batches of the 7 x 7 wgrad measured 7 % slower with it)
+template <int H, int W>
+constexpr bool use_progress_priority() {
+    return H * W >= 100;
+}
+
 // Four consecutive activations of type T as floats (one 16-byte or 8-byte global access).
 // Activations are touched exactly once per pass, so all global accesses are non-temporal:
 // outputs stream to HBM while the kernel runs instead of sitting dirty in L2 until the
@@ -609,7 +642,10 @@ __device__ __forceinline__ void run_canonical(const T *__restrict__ src, const f
     // Two register sets keep two batches in flight from HBM while a third is being computed.
     auto process = [&](auto &stg, int nb) {
         const int nvalid = n1 - nb;
+        if constexpr (use_progress_priority<H, W>())
+            set_progress_priority((nb - n0) / PB, (n1 - n0 + PB - 1) / PB);
         __syncthreads();  // previous batch fully consumed (first pass: zero fill done)
+        wait_vmem_done();
         if constexpr (PAIR)
             stg.template commit_pairs<GeoMap<G>, PLS, G::EH, G::EW>(lds, nvalid);
         else
@@ -705,7 +741,10 @@ __device__ __forceinline__ void run_table(const T *__restrict__ src, const float
     constexpr int R = H % 4 == 0 ? 4 : (H % 2 == 0 ? 2 : 1), HR = H / R;
     auto process = [&](auto &stg, int nb) {
         const int nvalid = n1 - nb;
+        if constexpr (use_progress_priority<H, W>())
+            set_progress_priority((nb - n0) / PB, (n1 - n0 + PB - 1) / PB);
         __syncthreads();
+        wait_vmem_done();
         stg.template commit<Map, PLS>(lds, nvalid);
         __syncthreads();
         if (nb + 2 * PB < n1)
@@ -958,7 +997,10 @@ __device__ __forceinline__ void run_canonical_wgrad(const T *__restrict__ x, con
         }
     auto process = [&](auto &stx, auto &stg, int nb) {
         const int nvalid = n1 - nb;
+        if constexpr (use_progress_priority<H, W>())
+            set_progress_priority((nb - n0) / PB, (n1 - n0 + PB - 1) / PB);
         __syncthreads();
+        wait_vmem_done();
         stx.template commit<GeoMap<G>, PLS>(lds, nvalid);
         stg.template commit<DyMap<W, DRS>, DYP>(ldy, nvalid);
         __syncthreads();
@@ -1051,7 +1093,10 @@ __device__ __forceinline__ void run_table_wgrad(const T *__restrict__ x, const T
     st.prefetch(xbase + (size_t)n0 * pstride, pstride, n1 - n0);
     for (int nb = n0; nb < n1; nb += PB) {
         const int nvalid = n1 - nb;
+        if constexpr (use_progress_priority<H, W>())
+            set_progress_priority((nb - n0) / PB, (n1 - n0 + PB - 1) / PB);
         __syncthreads();
+        wait_vmem_done();
         st.template commit<Map, PLS>(lds, nvalid);
         __syncthreads();
         if (nb + PB < n1) st.prefetch(xbase + (size_t)(nb + PB) * pstride, pstride, nvalid - PB);

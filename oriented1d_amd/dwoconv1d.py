@@ -159,8 +159,9 @@ def fprop(x, w, taps, stride=1, bias=None, nhwc=False):
     _check_taps(taps, C, K)
     b = f32_copy(bias) if bias is not None else None
     y = torch.empty(_out_shape(N, C, H, W, stride, nhwc), dtype=x.dtype, device=x.device)
-    _lib.check(lib.dwo_fprop(_ptr(x), _ptr(w2), _ptr(b), _ptr(taps), _ptr(y), N, C, H, W, K,
-                             stride, _DTYPES[x.dtype], int(nhwc), _stream(x)), "dwo_fprop")
+    _lib.check(_lib.launch(x.device, lib.dwo_fprop, _ptr(x), _ptr(w2), _ptr(b), _ptr(taps), _ptr(y),
+                           N, C, H, W, K, stride, _DTYPES[x.dtype], int(nhwc), _stream(x)),
+               "dwo_fprop")
     return y
 
 
@@ -176,8 +177,8 @@ def dgrad(dy, w, taps, in_hw, stride=1, nhwc=False):
     K = w2.shape[1]
     _check_taps(taps, C, K)
     dx = torch.empty((N, H, W, C) if nhwc else (N, C, H, W), dtype=dy.dtype, device=dy.device)
-    _lib.check(lib.dwo_dgrad(_ptr(dy), _ptr(w2), _ptr(taps), _ptr(dx), N, C, H, W, K, stride,
-                             _DTYPES[dy.dtype], int(nhwc), _stream(dy)), "dwo_dgrad")
+    _lib.check(_lib.launch(dy.device, lib.dwo_dgrad, _ptr(dy), _ptr(w2), _ptr(taps), _ptr(dx), N, C,
+                           H, W, K, stride, _DTYPES[dy.dtype], int(nhwc), _stream(dy)), "dwo_dgrad")
     return dx
 
 
@@ -197,8 +198,9 @@ def wgrad(dy, x, taps, K, stride=1, nhwc=False, with_bias=False):
     scratch = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=x.device)
     dw = torch.empty((C, 1, 1, K), dtype=torch.float32, device=x.device)
     db = torch.empty((C,), dtype=torch.float32, device=x.device) if with_bias else None
-    _lib.check(lib.dwo_wgrad(_ptr(dy), _ptr(x), _ptr(taps), _ptr(dw), _ptr(db), _ptr(scratch),
-                             nbytes, N, C, H, W, K, stride, dt, lay, _stream(x)), "dwo_wgrad")
+    _lib.check(_lib.launch(x.device, lib.dwo_wgrad, _ptr(dy), _ptr(x), _ptr(taps), _ptr(dw), _ptr(db),
+                           _ptr(scratch), nbytes, N, C, H, W, K, stride, dt, lay, _stream(x)),
+               "dwo_wgrad")
     return dw, db
 
 

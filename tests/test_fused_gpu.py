@@ -72,7 +72,8 @@ def test_nhwc_scale_add_nchw(N, C, H, W, with_scale, with_res, dtype):
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=["f32", "bf16", "f16"])
 @pytest.mark.parametrize("Cin,C,H,W,K,stride", [(3, 64, 64, 48, 31, 2), (3, 24, 37, 29, 15, 2),
-                                               (4, 8, 20, 20, 7, 1), (1, 16, 33, 70, 31, 4)])
+                                               (4, 8, 20, 20, 7, 1), (1, 16, 33, 70, 31, 4),
+                                               (3, 64, 224, 224, 31, 2)])  # the stem's own shape
 def test_pointwise_then_oriented_conv(oracle, Cin, C, H, W, K, stride, dtype):
     """dwo_pointwise_fprop_nhwc against the two separate layers: nn.Linear Cin -> C rounded to
     the activation type (what the reference's pw1 hands to dw1, models/convnext.py:177-178),

@@ -247,15 +247,76 @@ def test_randomized_shapes_all_paths(oracle, seed):
         _case(oracle, N, C, H, W, K, stride, dtype, nhwc, theta, seed=seed * 1000 + it)
 
 
-def test_wgrad_is_deterministic():
-    C, K = 96, 31
-    g = torch.Generator(device="cuda").manual_seed(5)
-    x = torch.randn(16, C, 56, 56, device="cuda", generator=g)
-    dy = torch.randn(16, C, 56, 56, device="cuda", generator=g)
+@pytest.mark.parametrize("nhwc", [False, True], ids=["nchw", "nhwc"])
+@pytest.mark.parametrize("C,HW", [(96, 56), (192, 28), (384, 14), (768, 7)])
+def test_wgrad_is_deterministic_on_both_reduction_paths(C, HW, nhwc):
+    """The partial sums of a channel are added in a fixed order, by the last workgroup of the
+    channel to finish (found through an integer counter) or by a second kernel: repeated calls
+    and the two paths must agree bit for bit, at the four stage shapes in both layouts."""
+    from oriented1d_amd import _lib
+
+    lib = _lib.ready(torch.device("cuda:0"))
+    K, N = 31, 32
+    g = torch.Generator(device="cuda").manual_seed(5 + HW)
+    shape = (N, HW, HW, C) if nhwc else (N, C, HW, HW)
+    x = torch.randn(shape, device="cuda", generator=g)
+    dy = torch.randn(shape, device="cuda", generator=g)
     taps = op.build_taps(torch.from_numpy(canonical_theta(C)), C, K).cuda()
-    a, adb = op.wgrad(dy, x, taps, K, with_bias=True)
-    b, bdb = op.wgrad(dy, x, taps, K, with_bias=True)
-    assert torch.equal(a, b) and torch.equal(adb, bdb)
+    print("determinism C%d %dx%d %s" % (C, HW, HW, "nhwc" if nhwc else "nchw"), flush=True)
+    a, adb = op.wgrad(dy, x, taps, K, nhwc=nhwc, with_bias=True)
+    for rep in range(4):
+        b, bdb = op.wgrad(dy, x, taps, K, nhwc=nhwc, with_bias=True)
+        assert torch.equal(a, b) and torch.equal(adb, bdb), rep
+    prev = lib.dwo_set_wgrad_reduction(0)  # second-kernel reduction
+    try:
+        assert prev == 1
+        c, cdb = op.wgrad(dy, x, taps, K, nhwc=nhwc, with_bias=True)
+        torch.cuda.synchronize()
+    finally:
+        lib.dwo_set_wgrad_reduction(1)
+    assert torch.equal(a, c) and torch.equal(adb, cdb)
+    d, ddb = op.wgrad(dy, x, taps, K, nhwc=nhwc, with_bias=True)  # the counters are back at zero
+    assert torch.equal(a, d) and torch.equal(adb, ddb)
+
+
+def test_wgrad_with_more_channels_than_a_counter_row(oracle):
+    """NCHW with more channels than a row of the library's counters holds (4096): the plane
+    kernel writes plain partial sums and the second kernel adds them."""
+    _case(oracle, 8, 4104, 7, 7, 31, 1, torch.float32, False, canonical_theta(4104), seed=4104)
+
+
+def test_wgrad_on_two_streams_at_once():
+    """Overlapping wgrad calls on two streams with their own scratch and outputs: each stream
+    counts on its own counters, so both give the single-stream result, call after call."""
+    from oriented1d_amd import _lib
+
+    _lib.ready(torch.device("cuda:0"))
+    C, K, HW, N = 192, 31, 28, 64
+    g = torch.Generator(device="cuda").manual_seed(9)
+    taps = op.build_taps(torch.from_numpy(canonical_theta(C)), C, K).cuda()
+    data = [(torch.randn(N, C, HW, HW, device="cuda", generator=g),
+             torch.randn(N, C, HW, HW, device="cuda", generator=g)) for _ in range(2)]
+    ref = [op.wgrad(dy, x, taps, K, with_bias=True) for x, dy in data]
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    got = [[], []]
+    for rep in range(12):
+        for k, st in enumerate(streams):
+            with torch.cuda.stream(st):
+                x, dy = data[k]
+                got[k].append(op.wgrad(dy, x, taps, K, with_bias=True))
+    torch.cuda.synchronize()
+    for k in range(2):
+        for dw, db in got[k]:
+            assert torch.equal(dw, ref[k][0]) and torch.equal(db, ref[k][1])
+
+
+@pytest.mark.parametrize("nhwc", [False, True], ids=["nchw", "nhwc"])
+def test_batch_128_bf16(oracle, nhwc):
+    """Batch 128, the batch the inference configuration runs at: all three operators of the
+    first stage's shape against the oracle."""
+    _case(oracle, 128, 96, 56, 56, 31, 1, torch.bfloat16, nhwc, grouped_theta(96), seed=128,
+          threads=min(16, oracle.max_threads()))
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
@@ -319,6 +380,7 @@ _TRAINING_LAUNCHES = [
     (2, 96, 128, 31, 1, False), (2, 192, 64, 31, 1, False), (2, 384, 32, 31, 1, False),
     (3, 768, 16, 31, 1, False),
     (1, 64, 512, 31, 2, True), (2, 64, 256, 31, 2, True), (2, 64, 224, 31, 2, True),
+    (2, 64, 112, 31, 2, True),  # second stem convolution of ConvNeXt-T-1D at 224 x 224
 ]
 
 
