@@ -33,7 +33,8 @@ def hipcc():
 
 PLANE_SHAPES = [(31, 56, 56), (31, 28, 28), (31, 14, 14), (31, 7, 7),
                 (15, 56, 56), (15, 28, 28), (15, 14, 14), (15, 7, 7),
-                (7, 56, 56), (7, 28, 28), (7, 14, 14)]  # = DWO_PLANE_SHAPES
+                (7, 56, 56), (7, 28, 28), (7, 14, 14),
+                (31, 64, 64), (31, 32, 32), (31, 16, 16)]  # = DWO_PLANE_SHAPES
 PLANE_TYPES = ["float", "bf16_t", "f16_t"]
 
 

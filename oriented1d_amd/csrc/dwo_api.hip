@@ -105,11 +105,13 @@ int try_plane_wgrad(const void *x, const void *dy, const void *taps, float *part
     return -100;
 }
 
+int nhwc_plane_batch(const ConvDims &d, int layout);
+
 // NHWC with the channel count a multiple of 4, stride 1, at the same extents: the slice kernels
 template <typename T>
 int try_nhwc_plane_conv(int op, const void *src, const float *w, const float *bias,
                         const void *taps, void *dst, const ConvDims &d, int layout, hipStream_t st) {
-    if (layout != DWO_NHWC || d.stride != 1 || d.C % kSliceCh != 0) return -100;
+    if (nhwc_plane_batch(d, layout) == 0) return -100;
 #define DWO_MATCH(K_, H_, W_)                                                                    \
     if (d.K == K_ && d.H == H_ && d.W == W_)                                                     \
         return launch_nhwc_plane_conv<T, K_, H_, W_>(op, src, w, bias, taps, dst, d.N, d.C, st);
@@ -134,7 +136,7 @@ bool nhwc_has_k(int K) {
 int nhwc_plane_batch(const ConvDims &d, int layout) {
     if (layout != DWO_NHWC || d.stride != 1 || d.C % kSliceCh != 0) return 0;
 #define DWO_MATCH(K_, H_, W_) \
-    if (d.K == K_ && d.H == H_ && d.W == W_) return NhwcTile<H_, W_>::PBI;
+    if (d.K == K_ && d.H == H_ && d.W == W_) return nhwc_plane_shape_rt(H_, W_) ? NhwcTile<H_, W_>::PBI : 0;
     DWO_PLANE_SHAPES(DWO_MATCH)
 #undef DWO_MATCH
     return 0;

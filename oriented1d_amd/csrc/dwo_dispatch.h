@@ -11,12 +11,14 @@
 // X(K, H, W): kernel size and plane extents with compile-time kernels (stride 1): the ConvNeXt
 // stage extents at 224 x 224 input for K = 31 (1D blocks, second conv of 1D++ blocks) and K = 15
 // (first conv of 1D++ blocks), and K = 7 at the three extents of the reference's own
-// micro-benchmark (analysis/benchmark.py:84-104)
+// micro-benchmark (analysis/benchmark.py:84-104); and the stage extents of a 512 x 512 input
+// that fit a workgroup's LDS (64, 32, 16 squared; NCHW only, see nhwc_plane_shape)
 #ifndef DWO_PLANE_SHAPES
 #define DWO_PLANE_SHAPES(X)                                   \
     X(31, 56, 56) X(31, 28, 28) X(31, 14, 14) X(31, 7, 7)     \
     X(15, 56, 56) X(15, 28, 28) X(15, 14, 14) X(15, 7, 7)     \
-    X(7, 56, 56) X(7, 28, 28) X(7, 14, 14)
+    X(7, 56, 56) X(7, 28, 28) X(7, 14, 14)                    \
+    X(31, 64, 64) X(31, 32, 32) X(31, 16, 16)
 #endif
 
 namespace dwo {

@@ -308,6 +308,9 @@ int launch_regplane_nhwc_conv(int op, const void *src, const float *w, const flo
 template <typename T, int K, int H, int W>
 int launch_nhwc_plane_conv(int op, const void *src, const float *w, const float *bias,
                            const void *taps, void *dst, int N, int C, hipStream_t st) {
+    if constexpr (!nhwc_plane_shape<H, W>()) {
+        return N == 0 ? 0 : -100;  // not built for this extent
+    } else {
     if constexpr (reg_plane_shape<H, W>()) {
         if (N > 0 && N <= 65535 && C % 32 == 0)
             return launch_regplane_nhwc_conv<T, K, H, W>(op, src, w, bias, taps, dst, N, C, st);
@@ -332,6 +335,7 @@ int launch_nhwc_plane_conv(int op, const void *src, const float *w, const float 
             (const T *)src, w, bias, taps, (T *)dst, N, C, groups);
     const hipError_t e = hipGetLastError();
     return e == hipSuccess ? 0 : (int)e;
+    }
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -653,6 +657,9 @@ template <typename T, int K, int H, int W>
 int launch_nhwc_plane_wgrad(const void *x, const void *dy, const void *taps, float *part, float *dw,
                             float *db, unsigned *tickets, int N, int C, int *groups_out,
                             hipStream_t st) {
+    if constexpr (!nhwc_plane_shape<H, W>()) {
+        return N == 0 ? 0 : -100;  // not built for this extent
+    } else {
     constexpr int NT = NhwcTile<H, W>::NT, PBI = NhwcTile<H, W>::PBI;
     const size_t lds = nhwc_plane_wgrad_lds_bytes<K, H, W>();
     static int cache[kMaxDevices];
@@ -668,6 +675,7 @@ int launch_nhwc_plane_wgrad(const void *x, const void *dy, const void *taps, flo
         (const T *)x, (const T *)dy, taps, WgradOut{part, dw, db, groups, tickets}, N, C);
     const hipError_t e = hipGetLastError();
     return e == hipSuccess ? 0 : (int)e;
+    }
 }
 
 }  // namespace dwo

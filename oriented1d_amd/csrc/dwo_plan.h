@@ -257,6 +257,18 @@ struct Tile<56, 56> {  // 784 / 448 / 448 items per plane
     static constexpr int LH = 4, LV = 7, LD = 8, PB = 1, NT = 448;
 };
 template <>
+struct Tile<64, 64> {  // 1024 / 1024 / 1152
+    static constexpr int LH = 4, LV = 4, LD = 4, PB = 1, NT = 512;
+};
+template <>
+struct Tile<32, 32> {  // 256 / 256 / 320
+    static constexpr int LH = 4, LV = 4, LD = 4, PB = 2, NT = 512;
+};
+template <>
+struct Tile<16, 16> {  // 64 / 64 / 96 (wgrad only: fprop and dgrad run on the register planes)
+    static constexpr int LH = 4, LV = 4, LD = 4, PB = 4, NT = 256;
+};
+template <>
 struct Tile<28, 28> {  // 196 / 196 / 224
     static constexpr int LH = 4, LV = 4, LD = 4, PB = 2, NT = 448;
 };
@@ -295,6 +307,16 @@ constexpr bool reg_plane_shape() {
 
 // NHWC slice kernels: a workgroup owns kSliceCh consecutive channels.
 constexpr int kSliceCh = 4;
+// Plane extents the NHWC slice kernels are built for (four haloed planes per image must fit a
+// workgroup's LDS next to the staging of their results); other extents run NHWC on the tile
+// kernels.
+constexpr bool nhwc_plane_shape_rt(int H, int W) {
+    return H == W && (H == 56 || H == 28 || H == 14 || H == 7);
+}
+template <int H, int W>
+constexpr bool nhwc_plane_shape() {
+    return nhwc_plane_shape_rt(H, W);
+}
 // Threads per workgroup and images staged per batch: the planes of a batch must fit in LDS, and
 // as many workgroups as possible should be resident per CU (at 14 x 14 one image per batch, four
 // workgroups per CU, measured 23 % faster than two images per batch and two workgroups).

@@ -119,6 +119,20 @@ def test_stage_shapes_reversed_orientations(oracle, C, HW, nhwc, dtype):
     _case(oracle, 2, C, HW, HW, 31, 1, dtype, nhwc, theta, seed=C + HW + 180)
 
 
+@pytest.mark.parametrize("dtype", DTYPES, ids=["f32", "bf16", "f16"])
+@pytest.mark.parametrize("C,HW", [(24, 64), (40, 32), (72, 16)])
+def test_stage_extents_of_a_512_input(oracle, C, HW, dtype):
+    """The stage extents of a 512 x 512 input that have compile-time planes (NCHW): canonical
+    angles round-robin and in groups, arbitrary angles mixed in, odd batch sizes that leave
+    partial batches and image groups; NHWC at the same extents (tile kernels)."""
+    rng = np.random.default_rng(HW)
+    _case(oracle, 9, C, HW, HW, 31, 1, dtype, False, canonical_theta(C), seed=HW * 7)
+    theta = grouped_theta(C, 0.5)
+    theta[2::5] = rng.uniform(-math.pi, 2 * math.pi, len(theta[2::5])).astype(np.float32)
+    _case(oracle, 5, C, HW, HW, 31, 1, dtype, False, theta, seed=HW * 7 + 1)
+    _case(oracle, 2, C, HW, HW, 31, 1, dtype, True, canonical_theta(C), seed=HW * 7 + 2)
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
 @pytest.mark.parametrize("C,HW", [(40, 56), (40, 28), (72, 14), (100, 7)])
 def test_stage_shapes_mixed_angles(oracle, C, HW, dtype):
