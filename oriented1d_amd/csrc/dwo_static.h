@@ -883,11 +883,20 @@ __device__ __forceinline__ void wgrad_finish(const WgradOut &out, float *lds, in
     // time).  Order is kept by completion instead: every thread waits until its stores are
     // acknowledged before the barrier that precedes the ticket, and the last workgroup's loads
     // are issued only after its ticket value has come back.
+    // (That argument rests on how gfx942 / gfx950 complete device-scope accesses -- stores
+    // written through and counted by vmcnt, loads served past the L2 of another XCD.  Any other
+    // target takes the ticket with release-acquire ordering, which the memory model itself
+    // guarantees.)
+#if defined(__gfx942__) || defined(__gfx950__)
+    constexpr int kTicketOrder = __ATOMIC_RELAXED;
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#else
+    constexpr int kTicketOrder = __ATOMIC_ACQ_REL;
+#endif
     __syncthreads();
     unsigned *flag = reinterpret_cast<unsigned *>(lds);
     if (threadIdx.x == 0)
-        *flag = __hip_atomic_fetch_add(out.tickets + ticket, 1u, __ATOMIC_RELAXED,
+        *flag = __hip_atomic_fetch_add(out.tickets + ticket, 1u, kTicketOrder,
                                        __HIP_MEMORY_SCOPE_AGENT);
     __syncthreads();
     if (*flag != (unsigned)out.NG - 1) return;

@@ -123,6 +123,45 @@ def test_network_matches_oracle_composition(oracle, variant):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("variant", ["1d", "1dpp"])
+def test_bf16_network_against_fp32_oracle_composition(oracle, variant):
+    """The 16-bit inference network (what the images-per-second figure runs) against an
+    independent result: the same weights in fp32 with every oriented convolution evaluated by
+    the oracle.  bf16 rounding accumulates over the layers, so the gate is 3e-2 of the output
+    scale (a wrong tap, weight or layout anywhere is an error of order one)."""
+    torch.manual_seed(7)
+    m = ConvNeXt1D(depths=(1, 2, 1, 1), dims=(16, 32, 64, 128), variant=variant, stem_dim1=24,
+                   num_classes=10, layer_scale_init_value=1.0).cuda().eval()
+    for name, p in m.named_parameters():
+        if name.endswith("bias"):
+            torch.nn.init.normal_(p, std=0.1)
+    x = torch.randn(2, 3, 64, 64, device="cuda")
+    import copy
+    m16 = copy.deepcopy(m).bfloat16()
+    with torch.no_grad():
+        y16 = m16(x.bfloat16()).float()
+
+    def oracle_forward(mod):
+        def fwd(t):
+            out = oracle.module_forward(t.detach().float().cpu().numpy(),
+                                        mod.weight.detach().float().cpu().numpy(),
+                                        mod.theta.detach().float().cpu().numpy(),
+                                        bias=mod.bias.detach().float().cpu().numpy(),
+                                        stride=mod.stride[0], nhwc=mod.nhwc,
+                                        resid=mod.resid is not None)
+            return torch.from_numpy(out).to(device=t.device, dtype=t.dtype)
+        return fwd
+
+    for mod in m.modules():
+        if isinstance(mod, DepthwiseOrientedConv1d):
+            mod.forward = oracle_forward(mod)
+    with torch.no_grad():
+        y_ref = m(x)
+    err = (y16 - y_ref).abs().max().item() / y_ref.abs().max().item()
+    assert y16.shape == (2, 10) and torch.isfinite(y16).all() and err < 3e-2, err
+
+
+@pytest.mark.gpu
 def test_training_step_and_stage_outputs():
     torch.manual_seed(1)
     m = ConvNeXt1D(depths=(1, 1, 1, 1), dims=(16, 32, 64, 128), variant="1dpp", stem_dim1=16,
