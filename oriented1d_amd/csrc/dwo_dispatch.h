@@ -25,27 +25,28 @@ namespace dwo {
 
 enum { OP_FPROP = 0, OP_DGRAD = 1 };
 
-// Image groups per channel.  A launch of C * g workgroups runs in rounds of `slots` resident
-// workgroups; the slowest workgroup of a round stages ceil(nbatch / g) batches, and a round that
-// fills only part of the slots runs its workgroups faster (one workgroup alone on a CU stages a
-// batch in about 0.55 of the time it takes next to two others).  The group count with the
-// smallest estimate wins, the smaller count on a tie: one full round at the stage shapes of
-// the networks (C * g = slots), two full rounds where C does not divide the slots (512 channels
-// on 768 slots: three groups, 1536 workgroups, instead of one group on two thirds of the slots).
+// Image groups per channel: as many workgroups as can be resident at once (no second round),
+// at most kMaxPlaneGroups and at most one staged batch per group.
 constexpr int kMaxPlaneGroups = 32;
 inline int plane_groups(int N, int C, int PB, int slots) {
+    int g = slots / C;
     const int nbatch = (N + PB - 1) / PB;
-    int best = 1;
-    double best_t = 1e30;
-    for (int g = 1; g <= nbatch && g <= kMaxPlaneGroups; g++) {
-        const long wgs = (long)C * g;
-        const int per = (nbatch + g - 1) / g;
-        const long full = wgs / slots, rest = wgs % slots;
-        double t = (double)full * per;
-        if (rest != 0) t += per * (0.55 + 0.45 * (double)rest / slots);
-        if (t < best_t - 1e-9) best_t = t, best = g;
+    if (g > nbatch) g = nbatch;
+    if (g > kMaxPlaneGroups) g = kMaxPlaneGroups;
+    if (g < 1) g = 1;
+    // A single round that would leave more than a quarter of the slots idle (512 channels on
+    // 768 slots): two full rounds of smaller workgroups instead, when C divides two rounds'
+    // worth of slots to within 5 %.
+    if ((long)C * g * 4 < (long)slots * 3) {
+        const int g2 = 2 * slots / C;
+        if (g2 > g && g2 <= nbatch && g2 <= kMaxPlaneGroups && (long)C * g2 * 20 >= (long)slots * 38)
+            return g2;
     }
-    return best;
+    // prefer an even split of the batches (every workgroup the same number of images) when one
+    // exists within 3/4 of the resident-slot count: the kernel ends with its slowest workgroup
+    for (int d = g; d * 4 >= g * 3 && d >= 1; d--)
+        if (nbatch % d == 0) return d;
+    return g;
 }
 
 template <typename T, int K, int H, int W>
