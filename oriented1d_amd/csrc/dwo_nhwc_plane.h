@@ -52,8 +52,25 @@ __device__ __forceinline__ unsigned rt_index(const GeoRt &g, unsigned r, unsigne
 // Workgroup id -> task (image group, channel slice), slices fastest.  Hardware deals
 // consecutive ids to the eight XCDs in turn; within every aligned block of 8*E tasks the order
 // is permuted so that the E slices of one 128-byte line get ids that land on one XCD.
+// When a pixel is not a whole number of lines (96 channels of a 16-bit type: 192 bytes) a line
+// holds slices of two pixels and no split of the slices keeps it on one XCD: then whole image
+// groups go to an XCD instead (group g to XCD g mod 8, all its slices with it), for as many
+// rounds of eight groups as there are.  (Measured at 96 x 56 x 56, bf16: 234 MB crossed the
+// fabric per fprop launch for 77 MB of tensors before this, every line fetched by three XCDs.)
 __device__ __forceinline__ void nhwc_task(int nslices, int groups, int E, int &slice, int &group) {
     const int id = blockIdx.x, total = nslices * groups, B = 8 * E;
+    if (nslices % E != 0) {
+        const int whole = (groups / 8) * 8 * nslices;  // tasks of whole rounds of eight groups
+        if (id < whole) {
+            const int j = id / 8;
+            group = id % 8 + 8 * (j / nslices);
+            slice = j % nslices;
+        } else {
+            slice = id % nslices;
+            group = id / nslices;
+        }
+        return;
+    }
     const int blk = id / B;
     int tau = id;
     if (blk * B + B <= total) {
