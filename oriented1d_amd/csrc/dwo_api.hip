@@ -557,13 +557,14 @@ int dwo_build_taps(const float *theta_host, int C, int K, void *taps_host) {
             if (c < C) order[placed++] = c;
         }
     }
-    // and the channels sorted by class: 0, .., 7, then the non-canonical ones (stable)
+    // and the channels sorted by the cost of their class in the plane kernels, dearest first:
+    // non-canonical (table-driven body), 22.5 and 157.5 degrees, 67.5 and 112.5, 0, 90, 45 and 135
+    // (stable within a class)
     int32_t *sorted = const_cast<int32_t *>(taps_sorted(taps_host, C, K));
-    for (int k = 0, placed = 0; k < 9; k++) {
-        const int want = k < 8 ? k : -1;
+    static const int by_cost[9] = {-1, 1, 7, 3, 5, 0, 4, 2, 6};
+    for (int k = 0, placed = 0; k < 9; k++)
         for (int c = 0; c < C; c++)
-            if (cls[c] == want) sorted[placed++] = c;
-    }
+            if (cls[c] == by_cost[k]) sorted[placed++] = c;
     hdr[7] = hdr[6] + (int32_t)taps_class_bytes(C);
     int8_t *extent = (int8_t *)taps_host + hdr[7];
     for (int c = 0; c < C; c++)

@@ -35,13 +35,14 @@ __device__ __forceinline__ lds_f2 lds_read2(const float *p) {
 //                              neighbouring workgroup ids (hence every XCD and CU) get a mix of
 //                              orientations
 //   int8  extent[C][2]         (max |dh|, max |dw|) over the channel's taps, padded to 16 bytes
-//   int32 sorted[C]            the channels sorted by orientation class (class 0, .., 7, then the
-//                              non-canonical ones): the per-channel workgroups of wgrad take
-//                              their channel from it, so that the workgroups sharing a CU run
-//                              the same class; padded to 16 bytes
+//   int32 sorted[C]            the channels sorted by what their orientation class costs in the
+//                              plane kernels, dearest first (non-canonical, 22.5 and 157.5
+//                              degrees, 67.5 and 112.5, 0, 90, 45 and 135): wgrad deals this
+//                              list to the CUs so that their loads come out even; padded to 16
+//                              bytes
 // ---------------------------------------------------------------------------------------------
 constexpr int32_t kTapsMagic = 0x44574f31;  // "DWO1"
-constexpr int32_t kTapsVersion = 5;
+constexpr int32_t kTapsVersion = 6;
 constexpr int kTapsHeaderInts = 8;
 constexpr int kTapsHeaderBytes = kTapsHeaderInts * 4;
 

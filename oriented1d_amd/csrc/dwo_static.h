@@ -411,19 +411,20 @@ __device__ __forceinline__ void plane_task(const void *blob, int C, int K, int g
     group = t / C;
 }
 // Workgroup -> (channel, image group) of wgrad.  Tasks are numbered channel-major over the tap
-// table's class-sorted channel list (a channel's image groups adjacent).  Workgroup ids b,
-// b + cus, b + 2 cus, .. meet on one CU (see above): those get consecutive tasks, i.e. the
-// workgroups that share a CU run the same orientation class, usually the same channel.  With
-// different classes on one CU the wgrad kernel measured 15 % slower at 56 x 56 (fprop and
-// dgrad measured the same or slightly better mixed, hence the two orders).  The host pads grids
-// above `cus` to a multiple of it; returns false for a padding workgroup.
+// table's cost-sorted channel list (most expensive orientation class first, a channel's image
+// groups adjacent).  Workgroup ids b, b + cus, b + 2 cus, .. meet on one CU (see above) and a
+// launch lasts as long as its most loaded CU, so the list is dealt to the CUs in rows of `cus`
+// tasks, every second row backwards: the CU that got the dearest task of one row gets the
+// cheapest of the next, and the sums per CU come out close to each other (class costs differ by
+// a quarter at 56 x 56).  The host pads grids above `cus` to a multiple of it; returns false for
+// a padding workgroup.
 __device__ __forceinline__ bool wgrad_task(const void *blob, int C, int K, int groups, int cus,
                                            int &c, int &group) {
     const int b = blockIdx.x, total = C * groups;
     int tau = b;
     if ((int)gridDim.x > cus) {
-        const int q = gridDim.x / cus;
-        tau = (b % cus) * q + b / cus;
+        const int row = b / cus, cu = b - row * cus;
+        tau = row * cus + ((row & 1) ? cus - 1 - cu : cu);
     }
     if (tau >= total) return false;
     c = taps_sorted(blob, C, K)[tau / groups];
