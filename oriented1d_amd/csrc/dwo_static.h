@@ -158,13 +158,27 @@ constexpr int table_pad() {
     return K / 2 < cmax(H, W) - 1 ? K / 2 : cmax(H, W) - 1;
 }
 
+// On planes wider and taller than K / 2 no tap of any angle can miss the plane (|dh|, |dw| <=
+// K / 2): the table bodies then run all K taps unrolled, lanes along consecutive outputs.
+template <int K, int H, int W>
+constexpr bool table_all_live() { return K / 2 < H && K / 2 < W; }
+// Row stride of the table bodies' staged plane: left margin (a multiple of four words), row,
+// right margin.  The unrolled bodies read one word per lane from consecutive outputs, which
+// wrap from one row to the next inside a wave: with a stride that equals W modulo the 32 banks
+// the wrapped lanes continue on the banks where the row left off (no conflicts at any offset).
+template <int K, int H, int W>
+constexpr int table_row_stride() {
+    constexpr int PAD = table_pad<K, H, W>(), PL = (PAD + 3) & ~3;
+    return table_all_live<K, H, W>() ? W + (PL + PAD + 31) / 32 * 32 : W + PL + PAD;
+}
+
 // orientation classes with a pair form (16-bit activations)
 constexpr bool pair_class(int cls) { return cls == CLS_H || cls == CLS_V; }
 
 template <int K, int H, int W, int... Os>
 constexpr int max_plane_floats(std::integer_sequence<int, Os...>) {
     constexpr int PAD = table_pad<K, H, W>();
-    int m = (H + 2 * PAD) * (W + 2 * PAD + 3);  // table-driven body
+    int m = (H + 2 * PAD) * cmax(W + 2 * PAD + 3, table_row_stride<K, H, W>());  // table-driven body
     ((m = cmax(m, Geo<Os, K, tile_L<H, W>(Os), H, W>::PLANE)), ...);
     ((m = cmax(m, Geo<Os, K, wgrad_L<H, W>(Os), H, W>::PLANE)), ...);
     // (pair geometries of the classes that have a pair form, see use_pairs)
@@ -697,12 +711,53 @@ template <int K, int H, int W>
 struct TableMap {
     static constexpr int PAD = table_pad<K, H, W>();
     static constexpr int PL = (PAD + 3) & ~3;
-    static constexpr int RS = W + PL + PAD;
+    static constexpr int RS = table_row_stride<K, H, W>();
     static constexpr bool kWide = RS % 4 == 0, kChunked = true;
     static __device__ __forceinline__ unsigned index(unsigned r, unsigned w) {
         return (r + PAD) * RS + w + PL;
     }
     static constexpr int step(int e) { return e; }
+};
+// The unrolled table bodies (table_all_live) keep the taps' LDS offsets (and, for fprop and
+// dgrad, weights) in scalar registers, and a thread evaluates table_rows outputs of one column,
+// H / table_rows rows apart, so one address per tap serves that many multiply-adds while
+// consecutive lanes still read consecutive words.
+template <int H, int W>
+constexpr int table_rows() {
+    // the divisor of H up to 8 that keeps most threads busy (the largest one among equals)
+    constexpr int PB = Tile<H, W>::PB, NT = Tile<H, W>::NT;
+    int best = 1;
+    long num = 0, den = 1;  // busy share of the best so far = num / den
+    for (int r = 1; r <= 8; r++) {
+        if (H % r != 0) continue;
+        const int items = PB * (H / r) * W, slots = (items + NT - 1) / NT * NT;
+        if ((long)items * den >= num * slots) best = r, num = items, den = slots;
+    }
+    return best;
+}
+// Taps of channel c for the unrolled table bodies: lane s of every wave holds tap s (LDS offset
+// and weight bits), and the bodies fetch tap s into scalar registers with a lane read when they
+// get to it.  (All K offsets and weights held in scalar registers for the whole body ran out of
+// them, and the few the compiler then parks in a vector register cost the canonical bodies
+// their last one.)
+template <class Map, int K>
+struct TableTaps {
+    static_assert(K <= 64, "one lane per tap");
+    int off, wbits;
+    __device__ __forceinline__ void load(const int8_t *__restrict__ dhdw, const float *__restrict__ wt,
+                                         int c, int sign) {
+        const int s = min((int)(threadIdx.x & 63), K - 1);
+        const int dh = dhdw[((size_t)c * K + s) * 2], dw = dhdw[((size_t)c * K + s) * 2 + 1];
+        off = sign * (dh * Map::RS + dw);
+        wbits = wt != nullptr ? __builtin_bit_cast(int, wt[(size_t)c * K + s]) : 0;
+    }
+    // (opaque to the optimiser: called once per batch, so that the lane reads stay inside the
+    // batch instead of being hoisted into 2 K scalar registers for the whole loop)
+    __device__ __forceinline__ void touch() { asm volatile("" : "+v"(off), "+v"(wbits)); }
+    __device__ __forceinline__ int offset(int s) const { return __builtin_amdgcn_readlane(off, s); }
+    __device__ __forceinline__ float weight(int s) const {
+        return __builtin_bit_cast(float, __builtin_amdgcn_readlane(wbits, s));
+    }
 };
 
 template <int OP, typename T, int K, int H, int W>
@@ -717,6 +772,74 @@ __device__ __forceinline__ void run_table(const T *__restrict__ src, const float
     static_assert((H + 2 * Map::PAD) * Map::RS <= PLS, "table body staging must fit the plane stride");
     const unsigned tid = threadIdx.x;
     const unsigned pstride = (unsigned)C * (H * W);
+    if constexpr (table_all_live<K, H, W>()) {
+        TableTaps<Map, K> taps;
+        taps.load(dhdw, wt, c, OP == OP_DGRAD ? -1 : 1);
+        const float bv = (OP == OP_FPROP && bias != nullptr) ? bias[c] : 0.f;
+        for (unsigned i = tid; i < PB * PLS; i += NT) lds[i] = 0.f;
+        const T *sbase = src + (size_t)c * (H * W);
+        T *dbase = dst + (size_t)c * (H * W);
+        constexpr int R = table_rows<H, W>(), HR = H / R;
+        constexpr int ITEMS = PB * HR * W, ITERS = (ITEMS + NT - 1) / NT;
+        auto process = [&](auto &stg, int nb) {
+            const int nvalid = n1 - nb;
+            taps.touch();
+            if constexpr (use_progress_priority<H, W>())
+                set_progress_priority((nb - n0) / PB, (n1 - n0 + PB - 1) / PB);
+            __syncthreads();
+            wait_vmem_done();
+            stg.template commit<Map, PLS>(lds, nvalid);
+            __syncthreads();
+            if (nb + 2 * PB < n1)
+                stg.prefetch(sbase + (size_t)(nb + 2 * PB) * pstride, pstride, nvalid - 2 * PB);
+            T *obase = dbase + (size_t)nb * pstride;
+#pragma unroll
+            for (int iter = 0; iter < ITERS; iter++) {
+                const unsigned f = tid + iter * NT;
+                const unsigned pl = f / (HR * W), g = f % (HR * W);
+                if (f < ITEMS && (int)pl < nvalid) {
+                    // (opaque: the K addresses base + offset are the same in every batch and
+                    // would otherwise be kept in K registers across the batch loop)
+                    unsigned at = pl * PLS + Map::index(g / W, g % W);
+                    asm volatile("" : "+v"(at));
+                    const float *base = lds + at;
+                    float acc[R];
+#pragma unroll
+                    for (int k = 0; k < R; k++) acc[k] = bv;
+                    // the reads of tap s + D are issued before the multiply-adds of tap s
+                    constexpr int D = R <= 4 ? 2 : 1;
+                    float v[D + 1][R];
+                    auto read_tap = [&](int s) {
+                        const float *q = base + taps.offset(s);
+#pragma unroll
+                        for (int k = 0; k < R; k++) v[s % (D + 1)][k] = q[k * (HR * Map::RS)];
+                    };
+#pragma unroll
+                    for (int s = 0; s < D && s < K; s++) read_tap(s);
+#pragma unroll
+                    for (int s = 0; s < K; s++) {
+                        if (s + D < K) read_tap(s + D);
+                        const float ws = taps.weight(s);
+#pragma unroll
+                        for (int k = 0; k < R; k++)
+                            acc[k] = __builtin_fmaf(v[s % (D + 1)][k], ws, acc[k]);
+                    }
+                    // (opaque to the optimiser: R store addresses kept as batch-loop invariants
+                    // would not fit the register budget next to the canonical bodies')
+                    unsigned o = pl * pstride + g;
+                    asm volatile("" : "+v"(o));
+#pragma unroll
+                    for (int k = 0; k < R; k++)
+                        st_out(obase + (o + k * (HR * W)), from_float<T>(acc[k]));
+                }
+            }
+        };
+        for (int nb = n0; nb < n1; nb += 2 * PB) {
+            process(sg.a, nb);
+            if (nb + PB < n1) process(sg.b, nb + PB);
+        }
+        return;
+    }
     // live taps of this channel as (LDS offset, weight) pairs (dead taps never reach the plane
     // and are skipped); kept in LDS behind the planes, read as one 8-byte broadcast per tap
     typedef int i2 __attribute__((ext_vector_type(2)));
@@ -1085,6 +1208,81 @@ __device__ __forceinline__ void run_table_wgrad(const T *__restrict__ x, const T
     constexpr int PLS = plane_floats<K, H, W>();
     const unsigned tid = threadIdx.x;
     const unsigned pstride = (unsigned)C * (H * W);
+    if constexpr (table_all_live<K, H, W>()) {
+        TableTaps<Map, K> taps;
+        taps.load(dhdw, nullptr, c, 1);
+        for (unsigned i = tid; i < PB * PLS; i += NT) lds[i] = 0.f;
+        float acc[K + 1];
+#pragma unroll
+        for (int s = 0; s <= K; s++) acc[s] = 0.f;
+        const T *xbase = x + (size_t)c * (H * W);
+        const T *gbase = dy + (size_t)c * (H * W);
+        constexpr int R = table_rows<H, W>(), HR = H / R;
+        constexpr int ITEMS = PB * HR * W, ITERS = (ITEMS + NT - 1) / NT;
+        Stager<T, H, W, PB, NT> st;
+        st.prefetch(xbase + (size_t)n0 * pstride, pstride, n1 - n0);
+        // dy of a batch goes straight from HBM to the registers of the lanes that use it, issued
+        // before the batch's x planes are written to LDS (a batch ahead, as for x, they would not
+        // fit next to the K + 1 sums)
+        for (int nb = n0; nb < n1; nb += PB) {
+            const int nvalid = n1 - nb;
+            taps.touch();
+            if constexpr (use_progress_priority<H, W>())
+                set_progress_priority((nb - n0) / PB, (n1 - n0 + PB - 1) / PB);
+            __syncthreads();
+            wait_vmem_done();
+            const T *gb = gbase + (size_t)nb * pstride;
+            T gy[ITERS][R];
+#pragma unroll
+            for (int iter = 0; iter < ITERS; iter++) {
+                const unsigned f = tid + iter * NT;
+                const unsigned pl = f / (HR * W), g = f % (HR * W);
+                const bool on = f < ITEMS && (int)pl < nvalid;
+                unsigned o = pl * pstride + g;  // (opaque: see the stores of run_table)
+                asm volatile("" : "+v"(o));
+#pragma unroll
+                for (int k = 0; k < R; k++)
+                    gy[iter][k] = on ? gb[o + k * (HR * W)] : from_float<T>(0.f);
+            }
+            st.template commit<Map, PLS>(lds, nvalid);
+            __syncthreads();
+            if (nb + PB < n1) st.prefetch(xbase + (size_t)(nb + PB) * pstride, pstride, nvalid - PB);
+#pragma unroll
+            for (int iter = 0; iter < ITERS; iter++) {
+                const unsigned f = tid + iter * NT;
+                const unsigned pl = f / (HR * W), g = f % (HR * W);
+                if (f < ITEMS && (int)pl < nvalid) {
+                    unsigned at = pl * PLS + Map::index(g / W, g % W);
+                    asm volatile("" : "+v"(at));  // (opaque: see run_table)
+                    const float *base = lds + at;
+                    float gf[R];
+#pragma unroll
+                    for (int k = 0; k < R; k++) gf[k] = to_float(gy[iter][k]);
+                    // the reads of tap s + D are issued before the multiply-adds of tap s
+                    constexpr int D = R <= 4 ? 2 : 1;
+                    float v[D + 1][R];
+                    auto read_tap = [&](int s) {
+                        const float *q = base + taps.offset(s);
+#pragma unroll
+                        for (int k = 0; k < R; k++) v[s % (D + 1)][k] = q[k * (HR * Map::RS)];
+                    };
+#pragma unroll
+                    for (int s = 0; s < D && s < K; s++) read_tap(s);
+#pragma unroll
+                    for (int s = 0; s < K; s++) {
+                        if (s + D < K) read_tap(s + D);
+#pragma unroll
+                        for (int k = 0; k < R; k++)
+                            acc[s] = __builtin_fmaf(v[s % (D + 1)][k], gf[k], acc[s]);
+                    }
+#pragma unroll
+                    for (int k = 0; k < R; k++) acc[K] += gf[k];
+                }
+            }
+        }
+        wgrad_epilogue<K, NT>(acc, lds, out, c, group, [](int s) { return s; });
+        return;
+    }
     int *toff = reinterpret_cast<int *>(lds + PB * PLS);  // LDS offset per tap; dead taps read the
     int *tlive = toff + K;                                 // centre and are zeroed at the end
     if (tid < K) {
