@@ -668,7 +668,7 @@ def main():
             for _ in range(2):
                 loss_ = train_step()
             torch.cuda.synchronize()
-            if not math.isfinite(float(loss_)) or not all(
+            if not math.isfinite(float(loss_.detach())) or not all(
                     bool(torch.isfinite(p_).all()) for p_ in net.parameters()):
                 raise RuntimeError("ConvNeXt-B-1D++ training step: non-finite loss or parameters")
             t0 = time.perf_counter()
@@ -699,7 +699,7 @@ def main():
             for _ in range(2):
                 loss_ = feature_step()
             torch.cuda.synchronize()
-            if not math.isfinite(float(loss_)) or not all(
+            if not math.isfinite(float(loss_.detach())) or not all(
                     p_.grad is None or bool(torch.isfinite(p_.grad).all()) for p_ in net.parameters()):
                 raise RuntimeError("ConvNeXt-T-1D features step: non-finite loss or gradients")
             t0 = time.perf_counter()

@@ -459,6 +459,17 @@ __device__ __forceinline__ void regplane_dispatch(const float *__restrict__ wt,
 #undef DWO_CASE
 }
 
+// Blocks of four images a wave of regplane_kernel works through.  The smallest planes have so
+// little arithmetic per block that one block per wave leaves every wave waiting out its own HBM
+// latency; the workgroup-barrier path (GroupPlanes) keeps one block.
+#ifndef DWO_REG_BLOCKS
+#define DWO_REG_BLOCKS 2
+#endif
+template <typename T, int H, int W>
+constexpr int reg_blocks_per_wave() {
+    return (!GroupIO<T, H, W>::kUse && H * W <= 64) ? DWO_REG_BLOCKS : 1;
+}
+
 template <int OP, typename T, int K, int H, int W>
 __global__ __launch_bounds__(kRegThreads) __attribute__((amdgpu_waves_per_eu(6, 8))) void regplane_kernel(
     const T *__restrict__ src, const float *__restrict__ wt, const float *__restrict__ bias,
@@ -467,7 +478,7 @@ __global__ __launch_bounds__(kRegThreads) __attribute__((amdgpu_waves_per_eu(6, 
     const int c = blockIdx.x * kRegWavesPerGroup + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     __shared__ __align__(16) float lds[kRegWavesPerGroup * RegIO<T, H, W>::kWaveFloats];
     float *wl = lds + (threadIdx.x >> 6) * RegIO<T, H, W>::kWaveFloats;
-    const int n0 = blockIdx.y * kRegPlanesPerWave;
+    const int n0 = blockIdx.y * kRegPlanesPerWave * reg_blocks_per_wave<T, H, W>();
     if constexpr (GroupIO<T, H, W>::kUse) {
         // (uniform over the grid: with whole channel blocks no wave leaves before the barriers)
         if (C % kRegWavesPerGroup == 0) {
@@ -481,11 +492,23 @@ __global__ __launch_bounds__(kRegThreads) __attribute__((amdgpu_waves_per_eu(6, 
         }
     }
     if (c >= C) return;  // whole wave; this path has no workgroup barriers
-    WavePlanes<T, H, W> pio;
-    pio.start(src, dst, c, C, n0, N - n0);
+    // kRegBlocksPerWave image blocks per wave, all fetched up front: the later blocks' HBM latency
+    // overlaps the earlier ones' arithmetic (the wave's LDS region is reused block after block;
+    // a wave's LDS operations complete in order)
+    constexpr int NB = reg_blocks_per_wave<T, H, W>();
+    WavePlanes<T, H, W> pio[NB];
+#pragma unroll
+    for (int q = 0; q < NB; q++)
+        if (n0 + q * kRegPlanesPerWave < N)
+            pio[q].start(src, dst, c, C, n0 + q * kRegPlanesPerWave, N - n0 - q * kRegPlanesPerWave);
     const int cls = __builtin_amdgcn_readfirstlane(taps_class(blob, C, K)[c]);
-    regplane_dispatch<OP, WavePlanes<T, H, W>, K, H, W>(wt, bias, blob, lds, wl, pio, c, cls, N - n0,
-                                                        (int)((threadIdx.x & 63) >> 4) < N - n0, true);
+#pragma unroll
+    for (int q = 0; q < NB; q++) {
+        const int left = N - n0 - q * kRegPlanesPerWave;
+        if (left > 0)
+            regplane_dispatch<OP, WavePlanes<T, H, W>, K, H, W>(
+                wt, bias, blob, lds, wl, pio[q], c, cls, left, (int)((threadIdx.x & 63) >> 4) < left, true);
+    }
 }
 
 // NHWC tensors, C a multiple of 32: workgroup = 32 channels of one image (NhwcLinePlanes)
@@ -528,8 +551,8 @@ template <typename T, int K, int H, int W>
 int launch_regplane_conv(int op, const void *src, const float *w, const float *bias,
                          const void *taps, void *dst, int N, int C, hipStream_t st) {
     if (N == 0) return 0;  // set-up only: nothing to prepare
-    const dim3 grid((C + kRegWavesPerGroup - 1) / kRegWavesPerGroup,
-                    (N + kRegPlanesPerWave - 1) / kRegPlanesPerWave),
+    constexpr int per_wave = kRegPlanesPerWave * reg_blocks_per_wave<T, H, W>();
+    const dim3 grid((C + kRegWavesPerGroup - 1) / kRegWavesPerGroup, (N + per_wave - 1) / per_wave),
         block(kRegThreads);
     if (grid.y > 65535) return -100;  // not covered: the dispatch goes on to the tile kernels
     if (op == OP_FPROP)
