@@ -520,10 +520,20 @@ __global__ __launch_bounds__(kRegThreads) __attribute__((amdgpu_waves_per_eu(DWO
     __shared__ __align__(16) float lds[kRegWavesPerGroup * PIO::kWaveFloats];
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     float *wl = lds + wave * PIO::kWaveFloats;
-    const int c0 = blockIdx.x * PIO::kBlockCh;
+    // Workgroup -> (channel block, image).  With 2-byte elements a block's pixel slices are half
+    // cache lines, and the other halves belong to the neighbouring channel block: hardware hands
+    // consecutive workgroup ids to the eight XCDs round-robin, so inside every aligned run of 16
+    // ids the two workgroups an XCD receives take neighbouring tasks, i.e. (with an even number
+    // of channel blocks) the two halves of the same lines, and the second one finds them in
+    // that XCD's L2.
+    unsigned task = blockIdx.x + blockIdx.y * gridDim.x;
+    if (sizeof(T) == 2 && (task | 15u) < gridDim.x * gridDim.y)
+        task = (task & ~15u) + 2 * (task & 7u) + ((task >> 3) & 1u);
+    const int block_x = task % gridDim.x, image = task / gridDim.x;
+    const int c0 = block_x * PIO::kBlockCh;
     const int c = c0 + wave + kRegWavesPerGroup * (int)((threadIdx.x & 63) >> 4);  // per 16-lane row
     PIO pio;
-    pio.start(src, dst, c0, C, blockIdx.y, kRegPlanesPerWave);
+    pio.start(src, dst, c0, C, image, kRegPlanesPerWave);
     // The straight-line bodies need one orientation per pass.  A wave whose four channels share
     // theirs (the usual case) makes one pass that also moves the planes; otherwise it moves them
     // itself and makes one pass per distinct class, each over the rows of that class only.
