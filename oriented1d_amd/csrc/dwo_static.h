@@ -428,7 +428,7 @@ __device__ __forceinline__ void plane_task(const void *blob, int C, int K, int g
 // table's cost-sorted channel list (most expensive orientation class first, a channel's image
 // groups adjacent).  Workgroup ids b, b + cus, b + 2 cus, .. meet on one CU (see above) and a
 // launch lasts as long as its most loaded CU, so the list is dealt to the CUs in rows of `cus`
-// tasks, every second row backwards: the CU that got the dearest task of one row gets the
+// tasks, every second row backwards: the CUs that got the dearest tasks of one row get the
 // cheapest of the next, and the sums per CU come out close to each other (class costs differ by
 // a quarter at 56 x 56).  The host pads grids above `cus` to a multiple of it; returns false for
 // a padding workgroup.
@@ -438,7 +438,11 @@ __device__ __forceinline__ bool wgrad_task(const void *blob, int C, int K, int g
     int tau = b;
     if ((int)gridDim.x > cus) {
         const int row = b / cus, cu = b - row * cus;
-        tau = row * cus + ((row & 1) ? cus - 1 - cu : cu);
+        // (backwards in blocks of eight: a task keeps its place modulo 8, i.e. its XCD, in every
+        // row, so channels that are neighbours in memory and share cache lines on the small
+        // planes still meet in one L2 when the class sizes are multiples of eight)
+        const int back = (cus & 7) == 0 ? cus - 8 - (cu & ~7) + (cu & 7) : cus - 1 - cu;
+        tau = row * cus + ((row & 1) ? back : cu);
     }
     if (tau >= total) return false;
     c = taps_sorted(blob, C, K)[tau / groups];
