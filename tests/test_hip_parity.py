@@ -145,6 +145,18 @@ def test_stage_shapes_mixed_angles(oracle, C, HW, dtype):
     _case(oracle, 3, C, HW, HW, 31, 1, dtype, False, grouped_theta(C, 0.5), seed=HW * 5)
 
 
+@pytest.mark.parametrize("dtype", DTYPES, ids=["f32", "bf16", "f16"])
+@pytest.mark.parametrize("K,HW", [(31, 56), (31, 28), (15, 56), (15, 14), (7, 28), (7, 14)])
+def test_arbitrary_angles_on_every_channel(oracle, K, HW, dtype):
+    """Every channel on the table-driven bodies (no canonical angle among them), on planes larger
+    than K / 2 in both directions, where those bodies run all K taps unrolled; batch sizes that
+    leave partial batches, angles on both sides of 180 degrees."""
+    rng = np.random.default_rng(K * 100 + HW)
+    theta = rng.uniform(-math.pi, 2 * math.pi, 11).astype(np.float32)
+    _case(oracle, 5, 11, HW, HW, K, 1, dtype, False, theta, seed=K + HW)
+    _case(oracle, 1, 11, HW, HW, K, 1, dtype, False, theta[::-1].copy(), seed=K + HW + 1)
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
 @pytest.mark.parametrize("C,HW", [(64, 14), (96, 7), (72, 14), (40, 7)])
 def test_nhwc_small_planes_mixed_classes(oracle, C, HW, dtype):
