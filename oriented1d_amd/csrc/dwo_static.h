@@ -722,10 +722,10 @@ struct TableMap {
     }
     static constexpr int step(int e) { return e; }
 };
-// The unrolled table bodies (table_all_live) keep the taps' LDS offsets (and, for fprop and
-// dgrad, weights) in scalar registers, and a thread evaluates table_rows outputs of one column,
-// H / table_rows rows apart, so one address per tap serves that many multiply-adds while
-// consecutive lanes still read consecutive words.
+// In the unrolled table bodies (table_all_live) a tap's LDS offset (and, for fprop and dgrad,
+// weight) is a scalar (TableTaps below), and a thread evaluates table_rows outputs of one
+// column, H / table_rows rows apart, so one address per tap serves that many multiply-adds
+// while consecutive lanes still read consecutive words.
 template <int H, int W>
 constexpr int table_rows() {
     // the divisor of H up to 8 that keeps most threads busy (the largest one among equals)
