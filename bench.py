@@ -78,7 +78,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--dtype", default="f32", choices=list(ELEM))
     ap.add_argument("--layout", default="nchw", choices=["nchw", "nhwc"])
-    ap.add_argument("--theta", default="roundrobin", choices=["roundrobin", "grouped"])
+    ap.add_argument("--theta", default="roundrobin", choices=["roundrobin", "grouped", "arbitrary"])
     ap.add_argument("--precondition-ms", type=float, default=60.0,
                     help="untimed steps run for this long before the warm-up steps, so that the "
                          "timed steps see the clocks of a continuous job")
@@ -135,6 +135,8 @@ def main():
     def theta_for(C, kind):
         if kind == "roundrobin":
             return np.array([(c % 8) * math.pi / 8 for c in range(C)], dtype=np.float32)
+        if kind == "arbitrary":  # no multiple of 22.5 degrees among them: the table-driven bodies
+            return np.array([0.1 + (c % 8) * 0.37 for c in range(C)], dtype=np.float32)
         return np.array([math.pi * (((8 * (c + 1) - 1) // C) / 8) for c in range(C)],
                         dtype=np.float32)
 
@@ -393,12 +395,14 @@ def main():
 
     # ------------------------------------------------------------------ the other rows
     # Same sweep in the other element type / layout / angle assignment (per-kernel times only,
-    # same launches per timing and repeats as the main table): bf16 NCHW, fp32 and bf16 NHWC-native, and fp32 NCHW with the networks'
-    # contiguous-group angles.
+    # same launches per timing and repeats as the main table): bf16 NCHW, fp32 and bf16 NHWC-native, fp32 NCHW with the networks'
+    # contiguous-group angles, and fp32 NCHW with angles that are no multiples of 22.5 degrees
+    # (every channel on the table-driven bodies).
     others = {}
     if not args.no_extra_sweeps and not args.only:
         for dt_, lay_, th_ in (("bf16", "nchw", "roundrobin"), ("f32", "nhwc", "roundrobin"),
-                               ("bf16", "nhwc", "roundrobin"), ("f32", "nchw", "grouped")):
+                               ("bf16", "nhwc", "roundrobin"), ("f32", "nchw", "grouped"),
+                               ("f32", "nchw", "arbitrary")):
             if (dt_, lay_, th_) == (args.dtype, args.layout, args.theta):
                 continue
             r = sweep(dt_, lay_, th_, 0, 0, args.kernel_iters, args.kernel_repeats)
