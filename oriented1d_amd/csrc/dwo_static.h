@@ -152,16 +152,21 @@ struct Vec4<f16_t> {
     }
 };
 
-// halo of the table-driven body: no live tap reaches further than this
+// The unrolled table bodies run all K taps of any angle, lanes along consecutive outputs.  The
+// staged plane then has a halo of K / 2 on every side, so that a tap that misses the plane
+// (|dh| >= H or |dw| >= W: small planes only) reads zeros like any tap that leaves it.  Used
+// where a batch of such planes stays within 40 KB of LDS (every plane extent of the build but
+// 7 x 7 at K = 31); elsewhere the halo stops at what a live tap can reach and the bodies loop
+// over the live taps.
+template <int K, int H, int W>
+constexpr bool table_unrolled() {
+    constexpr int PAD = K / 2, PL = (PAD + 3) & ~3;
+    return Tile<H, W>::PB * (H + 2 * PAD) * (W + (PL + PAD + 31) / 32 * 32) * 4 <= 40 * 1024;
+}
 template <int K, int H, int W>
 constexpr int table_pad() {
-    return K / 2 < cmax(H, W) - 1 ? K / 2 : cmax(H, W) - 1;
+    return table_unrolled<K, H, W>() || K / 2 < cmax(H, W) - 1 ? K / 2 : cmax(H, W) - 1;
 }
-
-// On planes wider and taller than K / 2 no tap of any angle can miss the plane (|dh|, |dw| <=
-// K / 2): the table bodies then run all K taps unrolled, lanes along consecutive outputs.
-template <int K, int H, int W>
-constexpr bool table_all_live() { return K / 2 < H && K / 2 < W; }
 // Row stride of the table bodies' staged plane: left margin (a multiple of four words), row,
 // right margin.  The unrolled bodies read one word per lane from consecutive outputs, which
 // wrap from one row to the next inside a wave: with a stride that equals W modulo the 32 banks
@@ -169,7 +174,7 @@ constexpr bool table_all_live() { return K / 2 < H && K / 2 < W; }
 template <int K, int H, int W>
 constexpr int table_row_stride() {
     constexpr int PAD = table_pad<K, H, W>(), PL = (PAD + 3) & ~3;
-    return table_all_live<K, H, W>() ? W + (PL + PAD + 31) / 32 * 32 : W + PL + PAD;
+    return table_unrolled<K, H, W>() ? W + (PL + PAD + 31) / 32 * 32 : W + PL + PAD;
 }
 
 // orientation classes with a pair form (16-bit activations)
@@ -722,7 +727,7 @@ struct TableMap {
     }
     static constexpr int step(int e) { return e; }
 };
-// In the unrolled table bodies (table_all_live) a tap's LDS offset (and, for fprop and dgrad,
+// In the unrolled table bodies (table_unrolled) a tap's LDS offset (and, for fprop and dgrad,
 // weight) is a scalar (TableTaps below), and a thread evaluates table_rows outputs of one
 // column, H / table_rows rows apart, so one address per tap serves that many multiply-adds
 // while consecutive lanes still read consecutive words.
@@ -744,16 +749,23 @@ constexpr int table_rows() {
 // get to it.  (All K offsets and weights held in scalar registers for the whole body ran out of
 // them, and the few the compiler then parks in a vector register cost the canonical bodies
 // their last one.)
-template <class Map, int K>
+template <class Map, int K, int H, int W>
 struct TableTaps {
     static_assert(K <= 64, "one lane per tap");
     int off, wbits;
+    // does tap s of channel c miss an H x W plane altogether?
+    static __device__ __forceinline__ bool dead(const int8_t *__restrict__ dhdw, int c, int s) {
+        const int dh = dhdw[((size_t)c * K + s) * 2], dw = dhdw[((size_t)c * K + s) * 2 + 1];
+        return dh >= H || dh <= -H || dw >= W || dw <= -W;
+    }
+    // (a tap that misses the plane reads the halo's zeros; its weight is zeroed as well, so that
+    // it adds nothing whatever the weight holds)
     __device__ __forceinline__ void load(const int8_t *__restrict__ dhdw, const float *__restrict__ wt,
                                          int c, int sign) {
         const int s = min((int)(threadIdx.x & 63), K - 1);
         const int dh = dhdw[((size_t)c * K + s) * 2], dw = dhdw[((size_t)c * K + s) * 2 + 1];
         off = sign * (dh * Map::RS + dw);
-        wbits = wt != nullptr ? __builtin_bit_cast(int, wt[(size_t)c * K + s]) : 0;
+        wbits = wt != nullptr && !dead(dhdw, c, s) ? __builtin_bit_cast(int, wt[(size_t)c * K + s]) : 0;
     }
     // (opaque to the optimiser: called once per batch, so that the lane reads stay inside the
     // batch instead of being hoisted into 2 K scalar registers for the whole loop)
@@ -776,8 +788,8 @@ __device__ __forceinline__ void run_table(const T *__restrict__ src, const float
     static_assert((H + 2 * Map::PAD) * Map::RS <= PLS, "table body staging must fit the plane stride");
     const unsigned tid = threadIdx.x;
     const unsigned pstride = (unsigned)C * (H * W);
-    if constexpr (table_all_live<K, H, W>()) {
-        TableTaps<Map, K> taps;
+    if constexpr (table_unrolled<K, H, W>()) {
+        TableTaps<Map, K, H, W> taps;
         taps.load(dhdw, wt, c, OP == OP_DGRAD ? -1 : 1);
         const float bv = (OP == OP_FPROP && bias != nullptr) ? bias[c] : 0.f;
         for (unsigned i = tid; i < PB * PLS; i += NT) lds[i] = 0.f;
@@ -1212,8 +1224,8 @@ __device__ __forceinline__ void run_table_wgrad(const T *__restrict__ x, const T
     constexpr int PLS = plane_floats<K, H, W>();
     const unsigned tid = threadIdx.x;
     const unsigned pstride = (unsigned)C * (H * W);
-    if constexpr (table_all_live<K, H, W>()) {
-        TableTaps<Map, K> taps;
+    if constexpr (table_unrolled<K, H, W>()) {
+        TableTaps<Map, K, H, W> taps;
         taps.load(dhdw, nullptr, c, 1);
         for (unsigned i = tid; i < PB * PLS; i += NT) lds[i] = 0.f;
         float acc[K + 1];
@@ -1284,7 +1296,11 @@ __device__ __forceinline__ void run_table_wgrad(const T *__restrict__ x, const T
                 }
             }
         }
-        wgrad_epilogue<K, NT>(acc, lds, out, c, group, [](int s) { return s; });
+        // (taps that miss the plane have summed halo zeros times dy: their gradient is zero by
+        // definition, whatever dy holds)
+        wgrad_epilogue<K, NT>(acc, lds, out, c, group, [&](int s) {
+            return TableTaps<Map, K, H, W>::dead(dhdw, c, s) ? -1 : s;
+        });
         return;
     }
     int *toff = reinterpret_cast<int *>(lds + PB * PLS);  // LDS offset per tap; dead taps read the

@@ -146,13 +146,17 @@ def test_stage_shapes_mixed_angles(oracle, C, HW, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=["f32", "bf16", "f16"])
-@pytest.mark.parametrize("K,HW", [(31, 56), (31, 28), (15, 56), (15, 14), (7, 28), (7, 14)])
+@pytest.mark.parametrize("K,HW", [(31, 56), (31, 28), (31, 14), (31, 7), (15, 56), (15, 14), (15, 7),
+                                  (7, 28), (7, 14)])
 def test_arbitrary_angles_on_every_channel(oracle, K, HW, dtype):
-    """Every channel on the table-driven bodies (no canonical angle among them), on planes larger
-    than K / 2 in both directions, where those bodies run all K taps unrolled; batch sizes that
-    leave partial batches, angles on both sides of 180 degrees."""
+    """Every channel on the table-driven bodies (no canonical angle among them): planes larger
+    than K / 2 in both directions, planes that some taps miss altogether (14 x 14 at K = 31,
+    7 x 7 at K = 15: angles next to 90 and 0 degrees are among the channels), and 7 x 7 at
+    K = 31, where the bodies loop over the live taps; batch sizes that leave partial batches,
+    angles on both sides of 180 degrees."""
     rng = np.random.default_rng(K * 100 + HW)
     theta = rng.uniform(-math.pi, 2 * math.pi, 11).astype(np.float32)
+    theta[:4] = np.float32([1.55, 1.62, 0.03, 3.1])  # steepest and flattest lines: the far taps leave a small plane
     _case(oracle, 5, 11, HW, HW, K, 1, dtype, False, theta, seed=K + HW)
     _case(oracle, 1, 11, HW, HW, K, 1, dtype, False, theta[::-1].copy(), seed=K + HW + 1)
 
