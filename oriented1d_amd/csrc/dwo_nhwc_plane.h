@@ -98,7 +98,7 @@ struct NhwcCtx {
     Vec4<T> pre[PF];
 
     __device__ __forceinline__ void zero_fill() {
-        for (unsigned i = threadIdx.x; i < kSliceCh * PBI * PLS; i += NT) lds[i] = 0.f;
+        lds_zero<NT>(lds, kSliceCh * PBI * PLS);
     }
     __device__ __forceinline__ void prefetch(int nb) {
         const T *base = src + (size_t)nb * HW * C;

@@ -196,6 +196,14 @@ constexpr int plane_floats() {
     return (max_plane_floats<K, H, W>(std::make_integer_sequence<int, 8>{}) + 3) & ~3;
 }
 
+// Zero `words` floats of LDS (a multiple of four, 16-byte aligned) with 16-byte writes.
+template <int NT>
+__device__ __forceinline__ void lds_zero(float *lds, unsigned words) {
+    typedef float f4 __attribute__((ext_vector_type(4)));
+    for (unsigned i = threadIdx.x * 4; i < words; i += NT * 4)
+        *reinterpret_cast<f4 *>(__builtin_assume_aligned(lds + i, 16)) = f4{0.f, 0.f, 0.f, 0.f};
+}
+
 // scalar stores of single results (4-byte ones non-temporal, like the vector stores)
 __device__ __forceinline__ void st_out(float *p, float v) { __builtin_nontemporal_store(v, p); }
 __device__ __forceinline__ void st_out(f16_t *p, f16_t v) { *p = v; }
@@ -609,7 +617,7 @@ __device__ __forceinline__ void run_canonical(const T *__restrict__ src, const f
     taps.load(wt, bias, c);
 
     // zero the staging area once; interiors are overwritten per batch, halos stay zero
-    for (unsigned i = tid; i < PB * PLS; i += NT) lds[i] = 0.f;
+    lds_zero<NT>(lds, PB * PLS);
 
     const T *sbase = src + (size_t)c * (H * W);
     T *dbase = dst + (size_t)c * (H * W);
@@ -792,7 +800,7 @@ __device__ __forceinline__ void run_table(const T *__restrict__ src, const float
         TableTaps<Map, K, H, W> taps;
         taps.load(dhdw, wt, c, OP == OP_DGRAD ? -1 : 1);
         const float bv = (OP == OP_FPROP && bias != nullptr) ? bias[c] : 0.f;
-        for (unsigned i = tid; i < PB * PLS; i += NT) lds[i] = 0.f;
+        lds_zero<NT>(lds, PB * PLS);
         const T *sbase = src + (size_t)c * (H * W);
         T *dbase = dst + (size_t)c * (H * W);
         constexpr int R = table_rows<H, W>(), HR = H / R;
@@ -873,7 +881,7 @@ __device__ __forceinline__ void run_table(const T *__restrict__ src, const float
         nlive_s = nl;
     }
     const float bv = (OP == OP_FPROP && bias != nullptr) ? bias[c] : 0.f;
-    for (unsigned i = tid; i < PB * PLS; i += NT) lds[i] = 0.f;
+    lds_zero<NT>(lds, PB * PLS);
     const T *sbase = src + (size_t)c * (H * W);
     T *dbase = dst + (size_t)c * (H * W);
     // A thread evaluates R outputs of one column, H / R rows apart: one tap read and one address
@@ -1125,15 +1133,10 @@ __device__ __forceinline__ void run_canonical_wgrad(const T *__restrict__ x, con
     constexpr int ITERS = (PB * G::IPP + NT - 1) / NT;
     const unsigned tid = threadIdx.x;
     const unsigned pstride = (unsigned)C * (H * W);
-    for (unsigned i = tid; i < PB * PLS; i += NT) lds[i] = 0.f;
     const T *xbase = x + (size_t)c * (H * W);
     const T *gbase = dy + (size_t)c * (H * W);
     float *ldy = lds + wgrad_dy_offset<K, H, W>();
     constexpr int DRS = dy_row_stride<G, W>(), DYP = wgrad_dy_plane<K, H, W>();
-
-    float acc[K + 1];  // acc[s] for representative taps s, acc[K] = sum of dy (bias gradient)
-#pragma unroll
-    for (int s = 0; s <= K; s++) acc[s] = 0.f;
 
     // DEPTH register sets per tensor keep that many batches in flight while another is summed.
     constexpr int DEPTH = H * W <= 256 ? DWO_WGRAD_DEPTH_SMALL : DWO_WGRAD_DEPTH;
@@ -1144,6 +1147,12 @@ __device__ __forceinline__ void run_canonical_wgrad(const T *__restrict__ x, con
             sx[k].prefetch(xbase + (size_t)(n0 + k * PB) * pstride, pstride, n1 - n0 - k * PB);
             sg[k].prefetch(gbase + (size_t)(n0 + k * PB) * pstride, pstride, n1 - n0 - k * PB);
         }
+    // (after the first loads are on their way: the zero fill runs under their latency)
+    lds_zero<NT>(lds, PB * PLS);
+
+    float acc[K + 1];  // acc[s] for representative taps s, acc[K] = sum of dy (bias gradient)
+#pragma unroll
+    for (int s = 0; s <= K; s++) acc[s] = 0.f;
     auto process = [&](auto &stx, auto &stg, int nb) {
         const int nvalid = n1 - nb;
         if constexpr (use_progress_priority<H, W>())
@@ -1227,7 +1236,7 @@ __device__ __forceinline__ void run_table_wgrad(const T *__restrict__ x, const T
     if constexpr (table_unrolled<K, H, W>()) {
         TableTaps<Map, K, H, W> taps;
         taps.load(dhdw, nullptr, c, 1);
-        for (unsigned i = tid; i < PB * PLS; i += NT) lds[i] = 0.f;
+        lds_zero<NT>(lds, PB * PLS);
         float acc[K + 1];
 #pragma unroll
         for (int s = 0; s <= K; s++) acc[s] = 0.f;
@@ -1311,7 +1320,7 @@ __device__ __forceinline__ void run_table_wgrad(const T *__restrict__ x, const T
         toff[tid] = dead ? 0 : dh * Map::RS + dw;
         tlive[tid] = dead ? -1 : (int)tid;
     }
-    for (unsigned i = tid; i < PB * PLS; i += NT) lds[i] = 0.f;
+    lds_zero<NT>(lds, PB * PLS);
     float acc[K + 1];
 #pragma unroll
     for (int s = 0; s <= K; s++) acc[s] = 0.f;
