@@ -97,6 +97,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra-sweeps", action="store_true",
                     help="skip the bf16 / NHWC / grouped-angle rows (other_configs)")
+    ap.add_argument("--arbitrary-row", action="store_true",
+                    help="add the other_configs row with angles that are no multiples of 22.5 degrees")
     ap.add_argument("--only", default="", help="restrict the per-kernel table, e.g. 96x56:fprop")
     ap.add_argument("--model-iters", type=int, default=5,
                     help="timed ConvNeXt-T-1D inference forwards (batch 128, bf16); 0 skips it")
@@ -396,13 +398,16 @@ def main():
     # ------------------------------------------------------------------ the other rows
     # Same sweep in the other element type / layout / angle assignment (per-kernel times only,
     # same launches per timing and repeats as the main table): bf16 NCHW, fp32 and bf16 NHWC-native, fp32 NCHW with the networks'
-    # contiguous-group angles, and fp32 NCHW with angles that are no multiples of 22.5 degrees
-    # (every channel on the table-driven bodies).
+    # contiguous-group angles, and, with --arbitrary-row, fp32 NCHW with angles that are no multiples of
+    # 22.5 degrees (every channel on the table-driven bodies; not in the default run: those launches
+    # carry the same kernel names and grids as the main sweep's and would blur a kernel trace of it).
     others = {}
     if not args.no_extra_sweeps and not args.only:
         for dt_, lay_, th_ in (("bf16", "nchw", "roundrobin"), ("f32", "nhwc", "roundrobin"),
                                ("bf16", "nhwc", "roundrobin"), ("f32", "nchw", "grouped"),
                                ("f32", "nchw", "arbitrary")):
+            if th_ == "arbitrary" and not args.arbitrary_row:
+                continue
             if (dt_, lay_, th_) == (args.dtype, args.layout, args.theta):
                 continue
             r = sweep(dt_, lay_, th_, 0, 0, args.kernel_iters, args.kernel_repeats)
